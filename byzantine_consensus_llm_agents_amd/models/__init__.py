@@ -8,6 +8,9 @@ def model_class(family: str):
     if family == "padadra":
         from .padadra import PadadraModel
         return PadadraModel
+    if family == "mabivik":
+        from .mabivik import MabivikModel
+        return MabivikModel
     from .transformer import DecoderModel
     return DecoderModel
 

@@ -378,6 +378,204 @@ class PadadraConfig:
         return n
 
 
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Softmax attention whose keys and values are read from one low-rank latent per token: the
+    cache holds the RMS-normed latent ``c`` (``kv_rank``) and one rotated key part (``rot_dim``)
+    shared by all heads; head h's unrotated key is ``W_uk[h] c`` (``dim``), its value ``W_uv[h] c``
+    (``vdim``).  Queries pass a latent of their own (``q_rank``).  Rotary (feature i pairs with
+    i + rot_dims / 2) acts on the first ``rot_dims`` features of the rotated part; ``rot_scaling``
+    = (factor, original, fast, slow) ramps the frequencies between two turn counts and multiplies
+    cos and sin by ``0.1 ln(factor) + 1``.  ``window`` keys are visible (0 = all); ``kv_from``: the
+    layer whose cache this one reads instead of holding one (-1 = its own)."""
+    heads: int
+    dim: int
+    rot_dim: int
+    vdim: int
+    q_rank: int
+    kv_rank: int
+    scale: float
+    window: int = 0
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    rot_scaling: Optional[tuple] = None
+    kv_from: int = -1
+
+    @property
+    def q_width(self) -> int:
+        return self.heads * (self.dim + self.rot_dim)
+
+    @property
+    def key_width(self) -> int:
+        """Cached key features per token: the latent and the shared rotated part."""
+        return self.kv_rank + self.rot_dim
+
+
+@dataclass(frozen=True)
+class HeadDeltaSpec:
+    """Gated delta rule with ONE decay per head: ``kv_heads`` q / k heads of ``dim``, ``heads``
+    value heads of ``vdim``, a short causal convolution of ``conv`` taps (0 = none) and silu on
+    q / k / v, a full-width silu output gate."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    conv: int = 0
+
+
+@dataclass(frozen=True)
+class SelectiveStateSpec:
+    """State-space mixer with a scalar decay per head (state ``state x vdim`` per head): one input
+    projection ``[z | x | B | C | dt]``, B and C shared by the heads of a group, a short causal
+    convolution with bias over x | B | C, the gated output RMS-normed in ``norm_groups`` parts."""
+    heads: int
+    vdim: int
+    state: int
+    groups: int = 1
+    conv: int = 0
+    norm_groups: int = 1
+
+    @property
+    def inner(self) -> int:
+        return self.heads * self.vdim
+
+    @property
+    def conv_channels(self) -> int:
+        return self.inner + 2 * self.groups * self.state
+
+
+@dataclass(frozen=True)
+class MabivikLayer:
+    type: str                    # "latent_attention" | "delta" | "mamba2"
+    mixer: object                # LatentAttentionSpec | HeadDeltaSpec | SelectiveStateSpec
+    mlp: Optional[FeedForwardSpec]
+
+
+@dataclass(frozen=True)
+class MabivikConfig:
+    """Mabivik: ``x <- x + post(mixer(pre(x)))`` then ``x <- x + post(ff(pre(x)))`` with dynamic-tanh
+    norms before and after every sublayer, a per-layer token input after the feed-forward
+    (``side_dim`` columns of a second embedding table per layer; 0 = none), mixers of three kinds
+    (latent attention, gated delta rule, selective state space) in the order the config lists,
+    mixture-of-experts feed-forwards whose experts come from a table row of the token id.
+    Everything is read from the model directory's config.json."""
+    name: str
+    hidden_size: int
+    vocab_size: int
+    layers: tuple
+    rms_eps: float = 1e-6
+    embed_scale: float = 1.0
+    logit_scale: float = 1.0
+    side_dim: int = 0
+    family: str = "mabivik"
+    max_position: int = 1 << 20
+    tie_embeddings: bool = False
+
+    @staticmethod
+    def _latent(m: dict, layers: list) -> LatentAttentionSpec:
+        rot = m.get("rot") or {}
+        sc = rot.get("scaling")
+        rot_dim = int(m.get("rot_dim", 0))
+        spec = LatentAttentionSpec(
+            heads=int(m["heads"]), dim=int(m["dim"]), rot_dim=rot_dim, vdim=int(m["vdim"]), q_rank=int(m["q_rank"]),
+            kv_rank=int(m["kv_rank"]), scale=float(m["scale"]), window=int((m.get("mask") or {}).get("size", 0)),
+            rot_dims=int(rot.get("dims", rot_dim)), rot_base=float(rot.get("base", 10000.0)),
+            rot_scaling=None if not sc else tuple(float(sc[k]) for k in ("factor", "original", "fast", "slow")),
+            kv_from=-1 if m.get("kv_from") is None else int(m["kv_from"]))
+        if spec.rot_dims % 2 or spec.rot_dims > spec.rot_dim:
+            raise ValueError("Mabivik: rot.dims even and <= rot_dim")
+        if spec.kv_from >= 0:
+            src = layers[spec.kv_from].mixer if spec.kv_from < len(layers) else None
+            if not isinstance(src, LatentAttentionSpec) or src.kv_from >= 0 or (src.kv_rank, src.rot_dim) != (spec.kv_rank, spec.rot_dim):
+                raise ValueError("Mabivik: kv_from names an earlier latent-attention layer with a cache of the same shape")
+        return spec
+
+    @classmethod
+    def from_dict(cls, c: dict, name: str = "mabivik") -> "MabivikConfig":
+        layers = []
+        for entry in c["layers"]:
+            m, kind = entry["mixer"], entry["type"]
+            if kind == "latent_attention":
+                mixer = cls._latent(m, layers)
+            elif kind == "delta":
+                mixer = HeadDeltaSpec(int(m["heads"]), int(m.get("kv_heads", m["heads"])), int(m["dim"]), int(m["vdim"]),
+                                      int(m.get("conv") or 0))
+                if mixer.heads % mixer.kv_heads:
+                    raise ValueError("Mabivik: heads must be a multiple of kv_heads")
+            elif kind == "mamba2":
+                mixer = SelectiveStateSpec(int(m["heads"]), int(m["vdim"]), int(m["state"]), int(m.get("groups", 1)),
+                                           int(m.get("conv") or 0), int(m.get("norm_groups", 1)))
+                if mixer.heads % mixer.groups or mixer.inner % mixer.norm_groups:
+                    raise ValueError("Mabivik: heads % groups, heads * vdim % norm_groups")
+            else:
+                raise ValueError(f"Mabivik: unknown layer type {kind!r}")
+            f = entry.get("mlp")
+            mlp = None
+            if f is not None:
+                if f.get("kind", "moe") != "moe":
+                    raise ValueError(f"Mabivik: unknown feed-forward kind {f['kind']!r}")
+                mlp = FeedForwardSpec("moe", int(f["expert"]["ff"]), int(f["router"]["experts"]), int(f["router"]["top"]))
+                if not 1 <= mlp.top <= mlp.experts:
+                    raise ValueError("Mabivik: router.top must be in [1, experts]")
+            layers.append(MabivikLayer(kind, mixer, mlp))
+        return cls(name=name, hidden_size=int(c["width"]), vocab_size=int(c["vocab"]), layers=tuple(layers),
+                   rms_eps=float(c["norm"]["eps"]), embed_scale=float((c.get("embedding") or {}).get("scale", 1.0)),
+                   logit_scale=float(c.get("logit_scale", 1.0)), side_dim=int((c.get("token_side") or {}).get("dim", 0)))
+
+    def to_dict(self) -> dict:
+        """The config.json form (inverse of `from_dict`)."""
+        out = []
+        for l in self.layers:
+            m = l.mixer
+            if l.type == "latent_attention":
+                mixer = {"heads": m.heads, "dim": m.dim, "rot_dim": m.rot_dim, "vdim": m.vdim, "q_rank": m.q_rank,
+                         "kv_rank": m.kv_rank, "scale": m.scale, "rot": {"dims": m.rot_dims, "base": m.rot_base}}
+                if m.rot_scaling:
+                    mixer["rot"]["scaling"] = dict(zip(("factor", "original", "fast", "slow"), m.rot_scaling))
+                if m.window:
+                    mixer["mask"] = {"size": m.window}
+                if m.kv_from >= 0:
+                    mixer["kv_from"] = m.kv_from
+            elif l.type == "delta":
+                mixer = {"heads": m.heads, "kv_heads": m.kv_heads, "dim": m.dim, "vdim": m.vdim}
+                if m.conv:
+                    mixer["conv"] = m.conv
+            else:
+                mixer = {"heads": m.heads, "vdim": m.vdim, "state": m.state, "groups": m.groups, "norm_groups": m.norm_groups}
+                if m.conv:
+                    mixer["conv"] = m.conv
+            mlp = None
+            if l.mlp is not None:
+                mlp = {"kind": "moe", "expert": {"ff": l.mlp.ff}, "router": {"experts": l.mlp.experts, "top": l.mlp.top}}
+            out.append({"type": l.type, "mixer": mixer, "mlp": mlp})
+        d = {"architecture": "Mabivik", "width": self.hidden_size, "vocab": self.vocab_size,
+             "embedding": {"scale": self.embed_scale}, "norm": {"eps": self.rms_eps}, "logit_scale": self.logit_scale,
+             "layers": out}
+        if self.side_dim:
+            d["token_side"] = {"dim": self.side_dim}
+        return d
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    def num_params(self) -> int:
+        W, n = self.hidden_size, 2 * self.vocab_size * self.hidden_size
+        for l in self.layers:
+            m = l.mixer
+            if l.type == "latent_attention":
+                n += W * m.q_rank + m.q_rank * m.q_width + m.heads * m.kv_rank * (m.dim + m.vdim) + 2 * W * m.heads * m.vdim
+                n += W * m.key_width if m.kv_from < 0 else 0
+            elif l.type == "delta":
+                n += W * (2 * m.kv_heads * m.dim + 3 * m.heads * m.vdim + 2 * m.heads)
+            else:
+                n += W * (2 * m.inner + 2 * m.groups * m.state + m.heads) + W * m.inner
+            if l.mlp is not None:
+                n += l.mlp.experts * 3 * W * l.mlp.ff
+            n += self.side_dim * (2 * W + self.vocab_size)
+        return n
+
+
 PRESETS = {
     "Qwen/Qwen3-8B": ModelConfig("Qwen/Qwen3-8B", "qwen3", 4096, 36, 32, 8, 128, 12288, 151936,
                                  qk_norm=True, max_position=40960),
@@ -415,6 +613,8 @@ def from_hf_config(path: str, name: Optional[str] = None):
         return MofidraConfig.from_dict(c, name or path)
     if str(c.get("architecture", "")).lower() == "padadra":
         return PadadraConfig.from_dict(c, name or path)
+    if str(c.get("architecture", "")).lower() == "mabivik":
+        return MabivikConfig.from_dict(c, name or path)
     arch = (c.get("model_type") or "").lower()
     family = "qwen3" if arch == "qwen3" else ("qwen2" if arch == "qwen2" else "mistral")
     heads = c["num_attention_heads"]

@@ -52,6 +52,17 @@ def _torch_ops() -> SimpleNamespace:
         delta_prepare=_ref.delta_prepare,
         gated_state_scan=_ref.gated_state_scan,
         head_norm_gate=_ref.head_norm_gate,
+        embed_scale_dyt=_ref.embed_scale_dyt,
+        residual_post_norm=_ref.residual_post_norm,
+        rmsnorm_cols=_ref.rmsnorm_cols,
+        latent_kv_write=_ref.latent_kv_write,
+        rope_half_tail=_ref.rope_half_tail,
+        head_linear=_ref.head_linear,
+        gate_mul=_ref.gate_mul,
+        ssm_prepare=_ref.ssm_prepare,
+        gated_group_norm=_ref.gated_group_norm,
+        moe_table_route=_ref.moe_table_route,
+        gelu_gather_mul=_ref.gelu_gather_mul,
         linear=torch.nn.functional.linear,
         rmsnorm=_ref.rmsnorm,
         add_rmsnorm=_ref.add_rmsnorm,

@@ -480,7 +480,8 @@ def moe_route(h, router_w, router_b, top: int, gate_w=None):
 
 def moe_experts(h, up, down, idx, weights, kind: str = "relu2"):
     """``sum_j weights[t, j] * down[e] act(up[e] h_t)``, e = idx[t, j]; up [E, ff, W],
-    down [E, W, ff].  Hidden activations are rounded to the activation dtype like a
+    down [E, W, ff].  kind "silu_gated": up is [E, 2 ff, W], rows [gate; up], and the hidden
+    activation is ``silu(gate h) * (up h)``.  Hidden activations are rounded to the activation dtype like a
     projection's output; the weighted sum is returned in fp32 (it goes into the fp32 residual)."""
     T, W = h.shape
     out = torch.zeros(T, W, dtype=torch.float32, device=h.device)
@@ -489,7 +490,13 @@ def moe_experts(h, up, down, idx, weights, kind: str = "relu2"):
         if rows.numel() == 0:
             continue
         x = h.index_select(0, rows)
-        y = torch.nn.functional.linear(act_fn(torch.nn.functional.linear(x, up[e]), kind), down[e])
+        z = torch.nn.functional.linear(x, up[e])
+        if kind == "silu_gated":
+            ff = z.shape[1] // 2
+            hid = (act_fn(z[:, :ff], "silu").float() * z[:, ff:].float()).to(z.dtype)
+        else:
+            hid = act_fn(z, kind)
+        y = torch.nn.functional.linear(hid, down[e])
         out.index_add_(0, rows, y.float() * weights[rows, slot][:, None])
     return out
 
@@ -552,10 +559,10 @@ def residual_mix_norm(x, normed, normed_scale: float, plain, mult: float, eps: f
     return rmsnorm_scalar(x, eps, gains, out_dtype)
 
 
-def short_conv(y, channels: int, w, meta, state, act=None):
+def short_conv(y, channels: int, w, meta, state, act=None, bias=None):
     """Causal convolution over time on the first ``channels`` columns of ``y`` [T, >= channels]:
-    ``out_t = sum_j w[:, j] u_(t - taps + 1 + j)`` (fp32 sum, rounded once), zeros before position
-    0, then ``act`` (None | "silu").  ``state`` [rows, taps - 1, channels]: the last inputs of
+    ``out_t = sum_j w[:, j] u_(t - taps + 1 + j)`` (+ ``bias`` fp32 [channels]; fp32 sum, rounded
+    once), zeros before position 0, then ``act`` (None | "silu").  ``state`` [rows, taps - 1, channels]: the last inputs of
     every state row; read where a segment reaches before its first row, then updated."""
     T, taps = y.shape[0], w.shape[1]
     u = y[:, :channels]
@@ -584,6 +591,8 @@ def short_conv(y, channels: int, w, meta, state, act=None):
             old = state[rows, (i + n).clamp(max=taps - 2)].float() * (pos0 > 0)[:, None]
             new[:, i] = torch.where((n >= b)[:, None], fresh, old)
         state[rows] = new.to(state.dtype)
+    if bias is not None:
+        acc = acc + bias.float()[None, :]
     if act == "silu":
         acc = acc * torch.sigmoid(acc)
     elif act is not None:
@@ -668,30 +677,33 @@ def hgrn2_prepare(y, off_q: int, off_f: int, heads: int, dim: int, f_bias, lower
 def delta_prepare(c, y, off_beta: int, a, a_log, dt_bias, heads: int, kv_heads: int, dim: int):
     """``c`` [T, >= 2 kv_heads dim]: q | k after convolution and activation; every q / k head
     becomes a unit vector ``x / sqrt(sum x^2 + 1e-6)`` (q also times dim^-1/2); ``beta = sigmoid(y
-    [:, off_beta + h])``; decay ``g = exp(-exp(a_log[h]) softplus(a + dt_bias))`` per head and key
-    channel (``a`` [T, heads dim]).  Returns fp32 (q [T, kv_heads, dim], k, g [T, heads, dim], beta [T, heads])."""
+    [:, off_beta + h])``; decay ``g = exp(-exp(a_log[h]) softplus(a + dt_bias))`` with ``a`` [T,
+    heads gd] (unit column stride), gd = dim (one decay per head and key channel) or 1 (one per
+    head).  Returns fp32 (q [T, kv_heads, dim], k, g [T, heads, gd], beta [T, heads])."""
     T, n = c.shape[0], kv_heads * dim
+    gd = a.shape[1] // heads
     q = c[:, :n].float().reshape(T, kv_heads, dim)
     k = c[:, n:2 * n].float().reshape(T, kv_heads, dim)
     q = q * torch.rsqrt(q.pow(2).sum(-1, keepdim=True) + 1e-6) * dim ** -0.5
     k = k * torch.rsqrt(k.pow(2).sum(-1, keepdim=True) + 1e-6)
     beta = torch.sigmoid(y[:, off_beta:off_beta + heads].float())
-    sp = torch.nn.functional.softplus(a.float() + dt_bias.float()).reshape(T, heads, dim)
+    sp = torch.nn.functional.softplus(a.float() + dt_bias.float()).reshape(T, heads, gd)
     g = torch.exp(-torch.exp(a_log.float())[None, :, None] * sp)
     return q, k, g, beta
 
 
 def gated_state_scan(q, k, g, v, beta, meta, state, delta: bool):
-    """Per head a ``dim x vdim`` fp32 state S with a decay per key channel, token after token:
+    """Per head a ``dim x vdim`` fp32 state S, token after token:
 
-        S <- diag(g_t) S;   u = v_t                      (delta False)
-                            u = beta_t (v_t - S^T k_t)   (delta True)
+        S <- diag(g_t) S;   u = v_t  (times beta_t when given)   (delta False)
+                            u = beta_t (v_t - S^T k_t)           (delta True)
         S <- S + k_t u^T;   o_t = S^T q_t
 
-    q / k [T, Gq, dim] fp32 (head h reads q / k head h // (H / Gq)), g [T, H, dim] fp32, v [T, H
-    vdim], beta [T, H] fp32 or None; ``state`` [rows, H, dim, vdim] fp32 is read (unless the
-    segment starts at position 0) and left at the segment's last token.  Returns fp32 o [T, H, vdim]."""
-    T, H, dim = g.shape
+    q / k [T, Gq, dim] fp32 (head h reads q / k head h // (H / Gq)), g fp32 [T, H, dim] (a decay
+    per key channel) or [T, H, 1] (one per head), v [T, H vdim], beta [T, H] fp32 or None;
+    ``state`` [rows, H, dim, vdim] fp32 is read (unless the segment starts at position 0) and left
+    at the segment's last token.  Returns fp32 o [T, H, vdim]."""
+    T, H = g.shape[:2]
     vdim = state.shape[3]
     per = H // q.shape[1]
     vf = v.float().reshape(T, H, vdim)
@@ -710,17 +722,173 @@ def gated_state_scan(q, k, g, v, beta, meta, state, delta: bool):
             u = vf[t]
             if delta:
                 u = beta[t][:, None] * (u - torch.einsum("hde,hd->he", S, kh[t]))
+            elif beta is not None:
+                u = beta[t][:, None] * u
             S = S + kh[t][:, :, None] * u[:, None, :]
             out[t] = torch.einsum("hde,hd->he", S, qh[t])
         state[rows[b]] = S
     return out
 
 
-def head_norm_gate(o, w, eps: float, gate, out_dtype):
+def head_norm_gate(o, w, eps: float, gate, out_dtype, gate_act: str = "sigmoid"):
     """o fp32 [T, H, vdim]: every head divided by its root mean square, times ``w`` [vdim], times
-    ``sigmoid(gate)`` (gate [T, H vdim] logits or None); returns [T, H vdim] in ``out_dtype``."""
+    ``sigmoid(gate)`` or ``silu(gate)`` (gate [T, H vdim] logits or None; ``gate_act``); returns
+    [T, H vdim] in ``out_dtype``."""
     T, H, vdim = o.shape
     y = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * w.float()
     if gate is not None:
-        y = y * torch.sigmoid(gate.float().reshape(T, H, vdim))
+        z = gate.float().reshape(T, H, vdim)
+        y = y * (torch.sigmoid(z) if gate_act == "sigmoid" else z * torch.sigmoid(z))
     return y.reshape(T, H * vdim).to(out_dtype)
+
+
+# ------------------------------------------------------------------ dynamic-tanh norms, latent attention, selective state
+# space, table-routed gated experts, per-layer token input (models/mabivik.py)
+#
+# A dynamic-tanh norm is the triple (alpha, w, b): ``tanh(alpha x) w + b`` elementwise (alpha a
+# number, w / b fp32 [W]); it takes no statistic of the row.  The latent-attention cache of one
+# layer is ``k : [num_blocks, 1, block_size, kv_rank + rot_dim]`` (the normed latent, then the
+# rotated shared key part) and ``v : [num_blocks, 1, kv_rank, block_size]`` (the latent again,
+# transposed per block): `multimap_attention` with one KV head reads them when every query
+# head carries ``W_uk[h]^T q_h`` in front of its rotated part, and its output is the softmax-
+# weighted latent, which ``W_uv[h]`` then expands.
+
+def dyt(x, norm, out_dtype):
+    """``tanh(alpha x) w + b`` in fp32, rounded once; ``norm`` = (alpha, w, b)."""
+    alpha, w, b = norm
+    return (torch.tanh(float(alpha) * x.float()) * w.float() + b.float()).to(out_dtype)
+
+
+def embed_scale_dyt(tokens, table, scale: float, norm, out_dtype):
+    """(fp32 stream ``scale * E[tokens]``, its `dyt` in ``out_dtype``)."""
+    x = table.index_select(0, tokens.long()).float() * scale
+    return x, dyt(x, norm, out_dtype)
+
+
+def residual_post_norm(x, y, post, pre, out_dtype):
+    """``x += post(y)`` in fp32, in place, with ``post`` = ("dyt", alpha, w, b) or ("rms", w, eps)
+    (``y / sqrt(mean(y^2) + eps) * w``); then returns what the next reader of x takes: ``pre`` =
+    ("dyt", alpha, w, b) -> `dyt` of the new x, ("copy",) -> x rounded to ``out_dtype``, None -> None."""
+    yf = y.float()
+    if post[0] == "dyt":
+        x.add_(torch.tanh(float(post[1]) * yf) * post[2].float() + post[3].float())
+    elif post[0] == "rms":
+        x.add_(yf * torch.rsqrt(yf.pow(2).mean(-1, keepdim=True) + float(post[2])) * post[1].float())
+    else:
+        raise ValueError(f"unknown post norm {post[0]!r}")
+    if pre is None:
+        return None
+    if pre[0] == "copy":
+        return x.to(out_dtype)
+    return dyt(x, pre[1:], out_dtype)
+
+
+def rmsnorm_cols(y, off: int, n: int, w, eps: float, out_dtype):
+    """RMS norm over the columns ``off : off + n`` of ``y`` (fp32), times ``w`` [n]; contiguous [T, n]."""
+    z = y[:, off:off + n].float()
+    return (z * torch.rsqrt(z.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(out_dtype)
+
+
+def ramp_inv_freq(dims: int, base: float, scaling=None, device=None):
+    """(fp32 frequencies [dims / 2], amplitude).  Plain: ``base^(-2i/dims)``, 1.  ``scaling`` =
+    (factor, original, fast, slow): with ``d(t) = dims ln(original / (2 pi t)) / (2 ln base)``, lo =
+    max(floor(d(fast)), 0), hi = min(ceil(d(slow)), dims - 1) and the ramp r_i = clamp((i - lo) /
+    max(hi - lo, 0.001), 0, 1) the frequency is ``f_i / factor * r_i + f_i (1 - r_i)`` and the
+    amplitude of cos and sin ``0.1 ln(factor) + 1``."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    f = float(base) ** (-2.0 * i / max(dims, 1))
+    amp = 1.0
+    if scaling is not None:
+        factor, orig, fast, slow = (float(v) for v in scaling)
+
+        def d(turns):
+            return dims * math.log(orig / (2.0 * math.pi * turns)) / (2.0 * math.log(base))
+        lo, hi = max(math.floor(d(fast)), 0), min(math.ceil(d(slow)), dims - 1)
+        r = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        f = f / factor * r + f * (1.0 - r)
+        amp = 0.1 * math.log(factor) + 1.0
+    return f.float().to(device), amp
+
+
+def _turn_half(x, positions, inv_freq, amp: float):
+    """x [T, ..., n]: feature i < len(inv_freq) pairs with i + len(inv_freq); cos and sin times amp."""
+    half = inv_freq.numel()
+    if not half:
+        return x
+    ang = positions.float().reshape(-1, *([1] * (x.dim() - 1))) * inv_freq.float()
+    c, s = ang.cos() * amp, ang.sin() * amp
+    a, b = x[..., :half], x[..., half:2 * half]
+    return torch.cat([a * c - b * s, b * c + a * s, x[..., 2 * half:]], dim=-1)
+
+
+def latent_kv_write(y, off: int, kv_rank: int, rot_dim: int, w, eps: float, positions, slots, inv_freq, amp: float,
+                    k_cache, v_cache):
+    """Columns ``off : off + kv_rank`` of ``y`` are RMS-normed (weight ``w``) into the latent c,
+    the next ``rot_dim`` are turned by the position (`_turn_half`, not normed); the token's cache
+    row becomes K = [c | turned part], V^T = c."""
+    c = rmsnorm_cols(y, off, kv_rank, w, eps, torch.float32)
+    kr = _turn_half(y[:, off + kv_rank:off + kv_rank + rot_dim].float(), positions, inv_freq, amp)
+    bs = k_cache.shape[2]
+    blk, o = (slots // bs).long(), (slots % bs).long()
+    k_cache[blk, 0, o] = torch.cat([c, kr], -1).to(k_cache.dtype)
+    v_cache[blk, 0, :, o] = c.to(v_cache.dtype)
+
+
+def rope_half_tail(src, src_off: int, dst, dst_off: int, positions, inv_freq, amp: float):
+    """``dst[:, h, dst_off:] = turn(src[:, h, src_off:])`` for every head of src [T, H, Ds] / dst
+    [T, H, Dd] (tails of equal width): the first ``2 len(inv_freq)`` features of the tail are turned
+    by the position (feature i pairs with i + half), the rest copied."""
+    dst[:, :, dst_off:] = _turn_half(src[:, :, src_off:].float(), positions, inv_freq, amp).to(dst.dtype)
+    return dst
+
+
+def head_linear(x3, w, out3=None):
+    """``out3[t, h] = w[h] x3[t, h]``: x3 [T, H, K] (any strides with a unit last one), w [H, N, K],
+    out3 [T, H, N] (a view to fill, or None: a new contiguous tensor)."""
+    if out3 is None:
+        out3 = torch.empty(x3.shape[0], x3.shape[1], w.shape[1], dtype=x3.dtype, device=x3.device)
+    torch.bmm(x3.transpose(0, 1), w.transpose(1, 2), out=out3.transpose(0, 1))
+    return out3
+
+
+def gate_mul(x, gate, kind: str):
+    """``x * sigmoid(gate)`` or ``x * silu(gate)`` (fp32, rounded once); gate [T, n] with any row stride."""
+    z = gate.float()
+    return (x.float() * (torch.sigmoid(z) if kind == "sigmoid" else z * torch.sigmoid(z))).to(x.dtype)
+
+
+def ssm_prepare(c, off_b: int, y, off_dt: int, dt_bias, a_log, heads: int, groups: int, state: int):
+    """``c`` [T, >= off_b + 2 groups state]: B | C after convolution and activation at ``off_b``;
+    ``dt = softplus(y[:, off_dt + h] + dt_bias[h])``, decay ``g = exp(-exp(a_log[h]) dt)``.  Returns
+    fp32 (C [T, groups, state], B [T, groups, state], g [T, heads, 1], dt [T, heads]): the read,
+    write and decay vectors of `gated_state_scan` and the scale of its written value."""
+    T, n = c.shape[0], groups * state
+    B = c[:, off_b:off_b + n].float().reshape(T, groups, state)
+    C = c[:, off_b + n:off_b + 2 * n].float().reshape(T, groups, state)
+    dt = torch.nn.functional.softplus(y[:, off_dt:off_dt + heads].float() + dt_bias.float())
+    g = torch.exp(-torch.exp(a_log.float())[None, :] * dt)
+    return C.contiguous(), B.contiguous(), g[:, :, None].contiguous(), dt.contiguous()
+
+
+def gated_group_norm(o, skip, skip_w, z, w, parts: int, eps: float, out_dtype):
+    """``u = (o + skip_w[h] skip) * silu(z)`` over o fp32 [T, H, vdim] (skip, z [T, H vdim], any row
+    stride), then u in ``parts`` equal pieces of the row, each divided by its own root mean
+    square, times ``w`` [H vdim]; returns [T, H vdim] in ``out_dtype``."""
+    T, H, vdim = o.shape
+    zf = z.float()
+    u = (o + skip_w.float()[None, :, None] * skip.float().reshape(T, H, vdim)).reshape(T, H * vdim) * (zf * torch.sigmoid(zf))
+    u = u.reshape(T, parts, -1)
+    u = u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps)
+    return (u.reshape(T, H * vdim) * w.float()).to(out_dtype)
+
+
+def moe_table_route(tokens, table, top: int):
+    """Experts by token id: (``table[token, :top]`` int32 [T, top], weights fp32 [T, top] = 1 / top)."""
+    idx = table.index_select(0, tokens.long())[:, :top].to(torch.int32).contiguous()
+    return idx, torch.full(idx.shape, 1.0 / top, dtype=torch.float32, device=idx.device)
+
+
+def gelu_gather_mul(z, tokens, table, off: int):
+    """``gelu_tanh(z) * table[token, off : off + n]`` for z [T, n] (fp32 math, rounded once)."""
+    e = table.index_select(0, tokens.long())[:, off:off + z.shape[1]].float()
+    return (act_fn(z.float(), "gelu_tanh") * e).to(z.dtype)
