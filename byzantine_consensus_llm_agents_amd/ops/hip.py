@@ -109,19 +109,36 @@ def load_library(path: str = None) -> ctypes.CDLL:
         "bcg_residual_mix_norm": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_float,
                                   c_float, c_float, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
         "bcg_short_conv": [c_void_p, c_int64, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                           c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+                           c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p],
         "bcg_rope_pairs_kv_write": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int,
                                     c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                     c_int, c_void_p],
         "bcg_rotate_pairs": [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
         "bcg_hgrn2_prepare": [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                               c_int, c_int, c_void_p],
-        "bcg_delta_prepare": [c_void_p, c_int64, c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                              c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "bcg_delta_prepare": [c_void_p, c_int64, c_void_p, c_int64, c_int, c_void_p, c_int64, c_int, c_void_p, c_void_p,
+                              c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
         "bcg_gated_state_scan": [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
-                                 c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
-        "bcg_head_norm_gate": [c_void_p, c_void_p, c_float, c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int,
+                                 c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "bcg_head_norm_gate": [c_void_p, c_void_p, c_float, c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                c_void_p],
+        "bcg_embed_scale_dyt": [c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                c_int, c_int, c_void_p],
+        "bcg_residual_post_norm": [c_void_p, c_void_p, c_int, c_int, c_float, c_void_p, c_void_p, c_float, c_int, c_float,
+                                   c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+        "bcg_rmsnorm_cols": [c_void_p, c_int64, c_int, c_int, c_void_p, c_float, c_void_p, c_int, c_int, c_void_p],
+        "bcg_latent_kv_write": [c_void_p, c_int64, c_int, c_int, c_int, c_void_p, c_float, c_void_p, c_void_p, c_void_p,
+                                c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+        "bcg_rope_half_tail": [c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_float, c_int,
+                               c_int, c_int, c_void_p],
+        "bcg_gate_mul": [c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_void_p],
+        "bcg_gated_act": [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p],
+        "bcg_ssm_prepare": [c_void_p, c_int64, c_int, c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                            c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+        "bcg_gated_group_norm": [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_float, c_void_p,
+                                 c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "bcg_gelu_gather_mul": [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p, c_int64, c_int, c_int, c_int,
+                                c_void_p],
         "bcg_moe_tile_rows": [],
         "bcg_moe_route": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                           c_int, c_int, c_void_p],
@@ -594,6 +611,8 @@ def hip_ops() -> SimpleNamespace:
     from .seqstate import seqstate_ops
     extra = seqmix_ops(lib, linear)
     extra.update(seqstate_ops(lib))
+    from .seqlatent import seqlatent_ops
+    extra.update(seqlatent_ops(lib))
 
     return SimpleNamespace(name="hip", **extra, rmsnorm_fp8=rmsnorm_fp8, embed_rmsnorm_fp8=embed_rmsnorm_fp8,
                            linear_fp8_residual=linear_fp8_residual, linear=linear, linear_silu=linear_silu, linear_residual=linear_residual,

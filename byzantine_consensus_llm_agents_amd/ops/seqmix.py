@@ -146,7 +146,8 @@ def seqmix_ops(lib, linear):
         dim = qd // maps
         G = k_cache.shape[1]
         NB, BS = _cache_ok(k_cache, v_cache, G, qd, vdim, q.dtype)
-        _req(H % G == 0 and maps in (1, 2) and dim <= 128 and vdim <= 256, "multimap attention: maps <= 2, dim <= 128, vdim <= 256")
+        _req(H % G == 0 and maps in (1, 2) and dim <= (256 if maps == 1 else 128) and vdim <= 256,
+             "multimap attention: maps <= 2, dim <= 128 (one map: 256), vdim <= 256")
         bt = meta.block_tables
         lens = meta.seq_lens if meta.attn_seq_lens is None else meta.attn_seq_lens
         _req(bt.dtype == torch.int32 and bt.dim() == 2 and bt.is_contiguous() and lens.dtype == torch.int32
@@ -204,10 +205,13 @@ def seqmix_ops(lib, linear):
 
     def moe_experts(h, up, down, idx, weights, kind="relu2"):
         T, W = h.shape
-        E, ff, _ = up.shape
+        E, n_up, _ = up.shape
         top = idx.shape[1]
-        _req(kind == "relu2", "moe_experts: relu2 experts")
-        _req(h.is_contiguous() and up.shape == (E, ff, W) and down.shape == (E, W, ff) and up.is_contiguous()
+        _req(kind in ("relu2", "silu_gated"), "moe_experts: relu2 or silu-gated experts")
+        gated = kind == "silu_gated"
+        _req(not gated or n_up % 2 == 0, "gated experts: [gate; up] rows")
+        ff = n_up // 2 if gated else n_up
+        _req(h.is_contiguous() and up.shape == (E, n_up, W) and down.shape == (E, W, ff) and up.is_contiguous()
              and down.is_contiguous() and up.dtype == h.dtype and down.dtype == h.dtype, "expert weights [E, ff, W] / [E, W, ff]")
         _req(idx.dtype == torch.int32 and idx.shape == (T, top) and idx.is_contiguous() and weights.dtype == torch.float32
              and weights.shape == (T, top) and weights.is_contiguous(), "routing tables [T, top]")
@@ -218,9 +222,16 @@ def seqmix_ops(lib, linear):
         sorted_ = torch.empty(cap, dtype=torch.int32, device=dev)
         tile_e = torch.empty(n_tiles, dtype=torch.int32, device=dev)
         _check(lib.bcg_moe_align(_p(idx), n_slots, E, _p(sorted_), cap, _p(tile_e), n_tiles, _stream()), "moe_align")
-        hidden = torch.empty(cap, ff, dtype=h.dtype, device=dev)
-        _check(lib.bcg_moe_gemm(_p(h), W, _p(up), _p(hidden), ff, _p(sorted_), _p(tile_e), n_tiles, ff, W, top, 1, 0, 1,
-                                f32, _stream()), "moe up")
+        if gated:   # the stacked projection, then silu(gate) * up over its halves
+            both = torch.empty(cap, n_up, dtype=h.dtype, device=dev)
+            _check(lib.bcg_moe_gemm(_p(h), W, _p(up), _p(both), n_up, _p(sorted_), _p(tile_e), n_tiles, n_up, W, top, 1, 0, 0,
+                                    f32, _stream()), "moe gate / up")
+            hidden = torch.empty(cap, ff, dtype=h.dtype, device=dev)
+            _check(lib.bcg_gated_act(_p(both), _p(hidden), cap, ff, f32, _stream()), "gated_act")
+        else:
+            hidden = torch.empty(cap, ff, dtype=h.dtype, device=dev)
+            _check(lib.bcg_moe_gemm(_p(h), W, _p(up), _p(hidden), ff, _p(sorted_), _p(tile_e), n_tiles, ff, W, top, 1, 0, 1,
+                                    f32, _stream()), "moe up")
         y = torch.empty(n_slots, W, dtype=h.dtype, device=dev)
         _check(lib.bcg_moe_gemm(_p(hidden), ff, _p(down), _p(y), W, _p(sorted_), _p(tile_e), n_tiles, W, ff, top, 0, 1, 0,
                                 f32, _stream()), "moe down")

@@ -79,7 +79,7 @@ def seqstate_ops(lib):
     def rmsnorm_scalar(x, eps, gains, out_dtype):
         return residual_mix_norm(x, [], 1.0, [], 0.0, eps, gains, out_dtype)
 
-    def short_conv(y, channels, w, meta, state, act=None):
+    def short_conv(y, channels, w, meta, state, act=None, bias=None):
         T = y.shape[0]
         _req(y.dim() == 2 and y.stride(1) == 1 and y.shape[1] >= channels, "short_conv: rows [T, >= channels], unit column stride")
         taps = w.shape[1]
@@ -91,11 +91,13 @@ def seqstate_ops(lib):
             _req(state is not None and state.dtype == y.dtype and state.is_contiguous() and state.dim() == 3
                  and state.shape[1:] == (taps - 1, channels), "conv state [rows, taps - 1, channels] in the activation dtype")
             rows = state.shape[0]
+        if bias is not None:
+            _f32(bias, channels, "convolution bias")
         out = torch.empty(T, channels, dtype=y.dtype, device=y.device)
         code = {None: 0, "silu": 1}[act]
         _check(lib.bcg_short_conv(_p(y), y.stride(0), channels, _p(w), taps, _p(meta.positions), _p(meta.token_seq),
-                                  _p(meta.q_start), _p(meta.state_rows), _p(state) if taps > 1 else None, rows, _p(out), code, T, B,
-                                  _act(y), _stream()), "short_conv")
+                                  _p(meta.q_start), _p(meta.state_rows), _p(state) if taps > 1 else None, rows, _p(out), code,
+                                  _p(bias), T, B, _act(y), _stream()), "short_conv")
         return out
 
     def rope_pairs_kv_write(qkv, positions, slots, n_q, n_kv, dim, vdim, q_norm, k_norm, eps, inv_freq, v_inv_freq,
@@ -151,39 +153,45 @@ def seqstate_ops(lib):
         T = c.shape[0]
         _req(c.dim() == 2 and c.stride(1) == 1 and c.shape[1] >= 2 * kv_heads * dim and y.dim() == 2 and y.stride(1) == 1
              and y.shape[0] == T and y.shape[1] >= off_beta + heads and c.dtype == y.dtype, "delta_prepare: rows q | k and beta")
-        _req(a.shape == (T, heads * dim) and a.is_contiguous() and a.dtype == c.dtype, "decay logits [T, heads dim]")
+        _req(a.dim() == 2 and a.shape[0] == T and a.shape[1] in (heads, heads * dim) and a.stride(1) == 1 and a.dtype == c.dtype,
+             "decay logits [T, heads dim] or [T, heads], unit column stride")
+        gd = a.shape[1] // heads
         _f32(a_log, heads, "A_log")
-        _f32(dt_bias, heads * dim, "dt_bias")
+        _f32(dt_bias, heads * gd, "dt_bias")
         _req(heads % kv_heads == 0 and heads <= 256, "heads % kv_heads, heads <= 256")
         dev = c.device
         q = torch.empty(T, kv_heads, dim, dtype=torch.float32, device=dev)
         k = torch.empty(T, kv_heads, dim, dtype=torch.float32, device=dev)
-        g = torch.empty(T, heads, dim, dtype=torch.float32, device=dev)
+        g = torch.empty(T, heads, gd, dtype=torch.float32, device=dev)
         beta = torch.empty(T, heads, dtype=torch.float32, device=dev)
-        _check(lib.bcg_delta_prepare(_p(c), c.stride(0), _p(y), y.stride(0), off_beta, _p(a), _p(a_log), _p(dt_bias), _p(q), _p(k),
-                                     _p(g), _p(beta), T, heads, kv_heads, dim, _act(c), _stream()), "delta_prepare")
+        _check(lib.bcg_delta_prepare(_p(c), c.stride(0), _p(y), y.stride(0), off_beta, _p(a), a.stride(0), gd, _p(a_log),
+                                     _p(dt_bias), _p(q), _p(k), _p(g), _p(beta), T, heads, kv_heads, dim, _act(c), _stream()),
+               "delta_prepare")
         return q, k, g, beta
 
     def gated_state_scan(q, k, g, v, beta, meta, state, delta):
-        T, H, dim = g.shape
-        _req(state.dim() == 4 and state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:3] == (H, dim),
+        T, H, gd = g.shape
+        _req(state.dim() == 4 and state.dtype == torch.float32 and state.is_contiguous() and state.shape[1] == H,
              "state fp32 [rows, H, dim, vdim]")
+        dim = state.shape[2]
+        _req(gd in (1, dim), "g fp32 [T, H, dim] or [T, H, 1]")
         vdim = state.shape[3]
         Gq = q.shape[1]
         for t, name in ((q, "q"), (k, "k")):
             _req(t.dtype == torch.float32 and t.is_contiguous() and t.shape == (T, Gq, dim), f"{name} fp32 [T, Gq, dim]")
         _req(g.dtype == torch.float32 and g.is_contiguous() and H % Gq == 0 and 1 <= dim <= 256, "g fp32 [T, H, dim], dim <= 256")
         _req(v.dim() == 2 and v.stride(1) == 1 and v.shape == (T, H * vdim), "v [T, H vdim], unit column stride")
-        if delta:
-            _req(beta is not None and beta.dtype == torch.float32 and beta.is_contiguous() and beta.shape == (T, H), "beta fp32 [T, H]")
+        _req(beta is not None or not delta, "the delta rule needs beta")
+        if beta is not None:
+            _req(beta.dtype == torch.float32 and beta.is_contiguous() and beta.shape == (T, H), "beta fp32 [T, H]")
         B = _segments(meta, T)
         out = torch.empty(T, H, vdim, dtype=torch.float32, device=g.device)
-        _check(lib.bcg_gated_state_scan(_p(q), _p(k), _p(g), _p(v), v.stride(0), _p(beta) if delta else None, _p(meta.positions),
+        _check(lib.bcg_gated_state_scan(_p(q), _p(k), _p(g), _p(v), v.stride(0), _p(beta), _p(meta.positions),
                                         _p(meta.q_start), _p(meta.state_rows), _p(state), state.shape[0], _p(out), B, H, Gq, dim,
-                                        vdim, int(bool(delta)), _act(v), _stream()), "gated_state_scan")
+                                        vdim, gd, int(bool(delta)), _act(v), _stream()), "gated_state_scan")
         return out
 
-    def head_norm_gate(o, w, eps, gate, out_dtype):
+    def head_norm_gate(o, w, eps, gate, out_dtype, gate_act="sigmoid"):
         _req(o.dim() == 3 and o.dtype == torch.float32 and o.is_contiguous(), "o fp32 [T, H, vdim]")
         T, H, vdim = o.shape
         _f32(w, vdim, "head norm weight")
@@ -193,8 +201,9 @@ def seqstate_ops(lib):
                  "gate logits [T, H vdim] in the activation dtype")
             stride = gate.stride(0)
         out = torch.empty(T, H * vdim, dtype=out_dtype, device=o.device)
-        _check(lib.bcg_head_norm_gate(_p(o), _p(w), eps, _p(gate), stride, _p(out), T, H, vdim, int(out_dtype == torch.float32),
-                                      _stream()), "head_norm_gate")
+        _check(lib.bcg_head_norm_gate(_p(o), _p(w), eps, _p(gate), stride, _p(out), T, H, vdim,
+                                      {"sigmoid": 0, "silu": 1}[gate_act], int(out_dtype == torch.float32), _stream()),
+               "head_norm_gate")
         return out
 
     return dict(embed_hashed_bigram_norm=embed_hashed_bigram_norm, residual_mix_norm=residual_mix_norm,

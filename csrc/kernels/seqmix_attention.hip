@@ -68,11 +68,11 @@ struct AttnArgs {
 // Everything that does not depend on the lane stays scalar: the page lookup and the slab base go
 // to SGPRs, a lane adds a 32-bit offset that is fixed for the whole loop.  Scores are kept in the
 // log2 domain (scale * log2 e folded into one multiply, v_exp_f32 directly).
-template <typename T, int KC, int VT, int KT, bool PF, bool FULL, int EXACT>
-__device__ __forceinline__ void attend_range(const AttnArgs& a_, int g, const typename Elem<T>::frag (&qf)[2][KC],
+template <typename T, int KC, int VT, int KT, bool PF, bool FULL, int EXACT, int NM>
+__device__ __forceinline__ void attend_range(const AttnArgs& a_, int g, const typename Elem<T>::frag (&qf)[NM][KC],
                                              int limit, int limit_min, int lo, int lo_max, int k_begin, int k_last,
-                                             const int* __restrict__ table, f32x4 (&acc)[2][VT], float (&mx)[2],
-                                             float (&den)[2]) {
+                                             const int* __restrict__ table, f32x4 (&acc)[NM][VT], float (&mx)[NM],
+                                             float (&den)[NM]) {
   typedef typename Elem<T>::frag F;
   // EXACT (1 or 2 = the number of maps): dim = 16 KC, vdim = 16 VT, 16-token pages, fragment-major slabs -- every guard
   // below is a compile-time constant, fragment offsets are immediates, the loop body is straight-line
@@ -113,13 +113,13 @@ __device__ __forceinline__ void attend_range(const AttnArgs& a_, int g, const ty
     page = (page < 0 || page >= a.num_blocks) ? 0 : page;
     return static_cast<size_t>(page) * a.G + g;
   };
-  auto load_k = [&](Cursor& c, F (&kf)[KT][2][KC]) {
+  auto load_k = [&](Cursor& c, F (&kf)[KT][NM][KC]) {
 #pragma unroll
     for (int u = 0; u < KT; ++u) {
       const T* kp = kc_base + slab_base(c) * k_slab + c.o * k_mul;
       step(c);
 #pragma unroll
-      for (int m = 0; m < 2; ++m)
+      for (int m = 0; m < NM; ++m)
 #pragma unroll
         for (int c2 = 0; c2 < KC; ++c2)
           kf[u][m][c2] = (m < a.maps && c2 < kc) ? load_frag_t<T, FULL>(kp + k_uni(m, c2) + k_lane, a.dim - (16 * c2 + 4 * grp), vec_k)
@@ -131,7 +131,7 @@ __device__ __forceinline__ void attend_range(const AttnArgs& a_, int g, const ty
   k_cur.p = k_begin / a.BS;
   k_cur.o = k_begin - k_cur.p * a.BS;
   v_cur = k_cur;
-  F kf[KT][2][KC];
+  F kf[KT][NM][KC];
   if (PF) load_k(k_cur, kf);
   for (int key0 = k_begin; key0 <= k_last; key0 += 16 * KT) {
     const T* vps[KT];
@@ -153,11 +153,11 @@ __device__ __forceinline__ void attend_range(const AttnArgs& a_, int g, const ty
       load_k(k_cur, kf);
     }
     // ---- S^T = K Q^T ----
-    f32x4 s[KT][2];
+    f32x4 s[KT][NM];
 #pragma unroll
     for (int u = 0; u < KT; ++u)
 #pragma unroll
-      for (int m = 0; m < 2; ++m) {
+      for (int m = 0; m < NM; ++m) {
         s[u][m] = f32x4{0.f, 0.f, 0.f, 0.f};
         if (m < a.maps) {
 #pragma unroll
@@ -170,9 +170,9 @@ __device__ __forceinline__ void attend_range(const AttnArgs& a_, int g, const ty
     if (PF && key0 + 16 * KT <= k_last) load_k(k_cur, kf);
     // ---- online softmax per query column; lane holds keys key0 + 16 u + 4 grp + i ----
     const bool masked = key0 + 16 * KT - 1 > limit_min || key0 < lo_max;   // (wave-uniform) some key of the iteration is hidden
-    F pf[KT][2];
+    F pf[KT][NM];
 #pragma unroll
-    for (int m = 0; m < 2; ++m) {
+    for (int m = 0; m < NM; ++m) {
       if (m >= a.maps) {
 #pragma unroll
         for (int u = 0; u < KT; ++u) pf[u][m] = zero_frag<T>();
@@ -221,12 +221,14 @@ __device__ __forceinline__ void attend_range(const AttnArgs& a_, int g, const ty
           F x;
           if constexpr (PF) x = vf[u][t]; else x = load_v(u, t);
           acc[0][t] = mma16(x, pf[u][0], acc[0][t]);
-          if (a.maps > 1) acc[1][t] = mma16(x, pf[u][1], acc[1][t]);
+          if constexpr (NM > 1) {
+            if (a.maps > 1) acc[1][t] = mma16(x, pf[u][1], acc[1][t]);
+          }
         }
   }
 }
 
-template <typename T, int KC, int VT, int KT, bool PF, bool FULL, int OCC, int EXACT = 0>
+template <typename T, int KC, int VT, int KT, bool PF, bool FULL, int OCC, int EXACT = 0, int NM = 2>
 __global__ __launch_bounds__(256, OCC) void prefill_kernel(AttnArgs a) {
   typedef typename Elem<T>::frag F;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -244,30 +246,39 @@ __global__ __launch_bounds__(256, OCC) void prefill_kernel(AttnArgs a) {
   const bool vec_k = a.vec_k && (a.dim & 3) == 0;
   const T* qrow = static_cast<const T*>(a.q) + (static_cast<size_t>(row) * a.H + h) * KD;
 
-  F qf[2][KC];
+  F qf[NM][KC];
 #pragma unroll
-  for (int m = 0; m < 2; ++m)
+  for (int m = 0; m < NM; ++m)
 #pragma unroll
     for (int c = 0; c < KC; ++c) {
       const int f = 16 * c + 4 * grp;
       qf[m][c] = (m < a.maps && c < kc) ? load_frag_t<T, FULL>(qrow + m * a.dim + f, a.dim - f, vec_k) : zero_frag<T>();
     }
-  f32x4 acc[2][VT];
+  f32x4 acc[NM][VT];
 #pragma unroll
-  for (int m = 0; m < 2; ++m)
+  for (int m = 0; m < NM; ++m)
 #pragma unroll
     for (int t = 0; t < VT; ++t) acc[m][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float mx[2] = {MAX_FLOOR, MAX_FLOOR}, den[2] = {0.f, 0.f};
+  float mx[NM], den[NM];
+#pragma unroll
+  for (int m = 0; m < NM; ++m) {
+    mx[m] = MAX_FLOOR;
+    den[m] = 0.f;
+  }
   if (a.sink != nullptr) {   // the sink starts the softmax: weight 1 at its own logit
     mx[0] = a.sink[h] * LOG2E;
     den[0] = 1.0f;
   }
   const int lo = a.window > 0 ? pos - a.window + 1 : 0, lo_max = a.window > 0 ? pos_max - a.window + 1 : 0;
   const int k_begin = a.window > 0 ? (max(0, pos_min - a.window + 1) & ~15) : 0;
-  attend_range<T, KC, VT, KT, PF, FULL, EXACT>(a, g, qf, pos, pos_min, lo, lo_max, k_begin, pos_max,
+  attend_range<T, KC, VT, KT, PF, FULL, EXACT, NM>(a, g, qf, pos, pos_min, lo, lo_max, k_begin, pos_max,
                                         a.block_tables + static_cast<size_t>(seq) * a.max_blocks, acc, mx, den);
   // ---- combine the maps, unit norm over the head's value features, store ----
-  const float i0 = 1.0f / den[0], i1 = a.maps > 1 ? a.lam / den[1] : 0.f;
+  const float i0 = 1.0f / den[0];
+  float i1 = 0.f;
+  if constexpr (NM > 1) {
+    if (a.maps > 1) i1 = a.lam / den[1];
+  }
   float ss = 0.f;
 #pragma unroll
   for (int t = 0; t < VT; ++t)
@@ -275,7 +286,9 @@ __global__ __launch_bounds__(256, OCC) void prefill_kernel(AttnArgs a) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         float o = acc[0][t][i] * i0;
-        if (a.maps > 1) o -= acc[1][t][i] * i1;
+        if constexpr (NM > 1) {
+          if (a.maps > 1) o -= acc[1][t][i] * i1;
+        }
         acc[0][t][i] = o;
         ss += o * o;   // rows >= vdim are zero (their V^T fragments were zero)
       }
@@ -301,7 +314,7 @@ __global__ __launch_bounds__(256, OCC) void prefill_kernel(AttnArgs a) {
 // head g (H / G) + 16 cg + c of the same token, so K and V^T are read once per KV head.  One wave
 // per (item, KV head x column group, SPLIT_KEYS-key split); partials as the merge kernel reads them
 // (running maxima in the log2 domain of `attend_range`).
-template <typename T, int KC, int VT, int KT, bool PF, bool FULL, int OCC, int EXACT = 0>
+template <typename T, int KC, int VT, int KT, bool PF, bool FULL, int OCC, int EXACT = 0, int NM = 2>
 __global__ __launch_bounds__(64, OCC) void decode_mfma_kernel(AttnArgs a) {
   typedef typename Elem<T>::frag F;
   const int lane = threadIdx.x, col = lane & 15, grp = lane >> 4;
@@ -321,32 +334,37 @@ __global__ __launch_bounds__(64, OCC) void decode_mfma_kernel(AttnArgs a) {
   const int kc = (a.dim + 15) >> 4, vt = (a.vdim + 15) >> 4;
   const bool vec_k = a.vec_k && (a.dim & 3) == 0;
   const T* qrow = static_cast<const T*>(a.q) + (static_cast<size_t>(row) * a.H + h) * KD;
-  F qf[2][KC];
+  F qf[NM][KC];
 #pragma unroll
-  for (int m = 0; m < 2; ++m)
+  for (int m = 0; m < NM; ++m)
 #pragma unroll
     for (int c = 0; c < KC; ++c) {
       const int f = 16 * c + 4 * grp;
       qf[m][c] = (m < a.maps && c < kc) ? load_frag_t<T, FULL>(qrow + m * a.dim + f, a.dim - f, vec_k) : zero_frag<T>();
     }
-  f32x4 acc[2][VT];
+  f32x4 acc[NM][VT];
 #pragma unroll
-  for (int m = 0; m < 2; ++m)
+  for (int m = 0; m < NM; ++m)
 #pragma unroll
     for (int t = 0; t < VT; ++t) acc[m][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float mx[2] = {MAX_FLOOR, MAX_FLOOR}, den[2] = {0.f, 0.f};
-  attend_range<T, KC, VT, KT, PF, FULL, EXACT>(a, g, qf, k_end - 1, k_end - 1, lo, lo, k_begin, k_end - 1,
+  float mx[NM], den[NM];
+#pragma unroll
+  for (int m = 0; m < NM; ++m) {
+    mx[m] = MAX_FLOOR;
+    den[m] = 0.f;
+  }
+  attend_range<T, KC, VT, KT, PF, FULL, EXACT, NM>(a, g, qf, k_end - 1, k_end - 1, lo, lo, k_begin, k_end - 1,
                                         a.block_tables + static_cast<size_t>(seq) * a.max_blocks, acc, mx, den);
   if (!col_ok) return;
   float* w = a.ws + ((static_cast<size_t>(item) * a.H + h) * a.n_splits + split) * (2 * a.maps + a.maps * a.vdim);
 #pragma unroll
-  for (int m = 0; m < 2; ++m)
+  for (int m = 0; m < NM; ++m)
     if (grp == 0 && m < a.maps) {
       w[m] = mx[m];
       w[a.maps + m] = den[m];
     }
 #pragma unroll
-  for (int m = 0; m < 2; ++m)
+  for (int m = 0; m < NM; ++m)
 #pragma unroll
     for (int t = 0; t < VT; ++t)
       if (m < a.maps && t < vt) {
@@ -435,8 +453,10 @@ int launch_prefill(const AttnArgs& a, int n_tiles, int tile_rows, hipStream_t s)
   if (small) {
     if (full) prefill_kernel<T, 4, 8, 1, false, true, 2><<<grid, 256, 0, s>>>(a);
     else prefill_kernel<T, 4, 8, 1, false, false, 2><<<grid, 256, 0, s>>>(a);
-  } else {   // (the branch-free form of the wide instance runs out of registers)
+  } else if (a.dim <= 128) {   // (the branch-free form of the wide instance runs out of registers)
     prefill_kernel<T, 8, 16, 1, false, false, 1><<<grid, 256, 0, s>>>(a);
+  } else {   // one map of up to 256 key features (a latent plus a rotated part)
+    prefill_kernel<T, 16, 16, 1, false, false, 1, 0, 1><<<grid, 256, 0, s>>>(a);
   }
   return BCG_CHECK_LAUNCH();
 }
@@ -476,8 +496,10 @@ int launch_decode(const AttnArgs& a, int n_items, hipStream_t s) {
   } else if (a.dim <= 64 && a.vdim <= 128) {
     if (full) decode_mfma_kernel<T, 4, 8, 1, false, true, 2><<<grid, 64, 0, s>>>(a);
     else decode_mfma_kernel<T, 4, 8, 1, false, false, 2><<<grid, 64, 0, s>>>(a);
-  } else {
+  } else if (a.dim <= 128) {
     decode_mfma_kernel<T, 8, 16, 1, false, false, 1><<<grid, 64, 0, s>>>(a);
+  } else {
+    decode_mfma_kernel<T, 16, 16, 1, false, false, 1, 0, 1><<<grid, 64, 0, s>>>(a);
   }
   if (a.vdim <= 128) decode_merge_kernel<T, 2><<<dim3(a.H, n_items), 64, 0, s>>>(a);
   else decode_merge_kernel<T, 4><<<dim3(a.H, n_items), 64, 0, s>>>(a);
@@ -497,7 +519,7 @@ BCG_API int bcg_multimap_attention(int mode, const void* q, const void* k_cache,
                                    float out_scale, int tile_rows, int is_f32, int window, const void* sink, void* stream) {
   if (n_work <= 0) return 0;
   if ((window > 0 || sink != nullptr) && maps != 1) return -2;
-  if (maps < 1 || maps > 2 || dim > 128 || vdim > 256 || BS % 16 || H % G || n_work > 65535 * 16) return -2;
+  if (maps < 1 || maps > 2 || dim > (maps == 1 ? 256 : 128) || vdim > 256 || BS % 16 || H % G || n_work > 65535 * 16) return -2;
   AttnArgs a;
   a.q = q; a.k_cache = k_cache; a.v_cache = v_cache;
   a.block_tables = static_cast<const int*>(block_tables); a.q_start = static_cast<const int*>(q_start);

@@ -142,20 +142,21 @@ __global__ __launch_bounds__(NT) void residual_mix_norm_kernel(float* __restrict
 }
 
 // ---------------------------------------------------------------- short causal convolution over time
-// out[t, c] = act(sum_j w[c, j] u(pos_t - taps + 1 + j)[c]); u before the segment comes from the
+// out[t, c] = act(bias[c] + sum_j w[c, j] u(pos_t - taps + 1 + j)[c]) (bias null: none); u before the segment comes from the
 // state row (its last taps - 1 inputs, oldest first), u before position 0 is zero.
 template <typename T>
 __global__ __launch_bounds__(NT) void short_conv_kernel(const T* __restrict__ y, int64_t y_stride, int C,
                                                         const float* __restrict__ w, int taps,
                                                         const int* __restrict__ positions, const int* __restrict__ token_seq,
                                                         const int* __restrict__ q_start, const int* __restrict__ state_rows,
-                                                        const T* __restrict__ state, int n_rows, T* __restrict__ out, int act) {
+                                                        const T* __restrict__ state, int n_rows, T* __restrict__ out, int act,
+                                                        const float* __restrict__ bias) {
   const int t = blockIdx.x, c = blockIdx.y * NT + threadIdx.x;
   if (c >= C) return;
   const int seg = token_seq[t], off = t - q_start[seg], pos = positions[t];
   const int sr = state_rows[seg];
   const bool row_ok = sr >= 0 && sr < n_rows;
-  float acc = 0.f;
+  float acc = bias != nullptr ? bias[c] : 0.f;
   for (int j = 0; j < taps; ++j) {
     const int back = taps - 1 - j;
     float u = 0.f;
@@ -177,15 +178,18 @@ __global__ __launch_bounds__(NT) void short_conv_vec_kernel(const T* __restrict_
                                                             const float* __restrict__ w, const int* __restrict__ positions,
                                                             const int* __restrict__ token_seq, const int* __restrict__ q_start,
                                                             const int* __restrict__ state_rows, const T* __restrict__ state,
-                                                            int n_rows, T* __restrict__ out, int act, int T_) {
+                                                            int n_rows, T* __restrict__ out, int act, int T_,
+                                                            const float* __restrict__ bias) {
   struct alignas(sizeof(T) * VEC) Vec { T e[VEC]; };
   const int c = (blockIdx.y * NT + threadIdx.x) * VEC;
   if (c >= C) return;
-  float wr[VEC][TAPS];
+  float wr[VEC][TAPS], br[VEC];
 #pragma unroll
-  for (int e = 0; e < VEC; ++e)
+  for (int e = 0; e < VEC; ++e) {
+    br[e] = bias != nullptr ? bias[c + e] : 0.f;
 #pragma unroll
     for (int j = 0; j < TAPS; ++j) wr[e][j] = w[static_cast<size_t>(c + e) * TAPS + j];
+  }
   const int t_end = min(T_, (static_cast<int>(blockIdx.x) + 1) * CONV_ROWS);
   for (int t = blockIdx.x * CONV_ROWS; t < t_end; ++t) {
     const int seg = token_seq[t], off = t - q_start[seg], pos = positions[t];
@@ -193,7 +197,7 @@ __global__ __launch_bounds__(NT) void short_conv_vec_kernel(const T* __restrict_
     const bool row_ok = sr >= 0 && sr < n_rows;
     float acc[VEC];
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+    for (int e = 0; e < VEC; ++e) acc[e] = br[e];
 #pragma unroll
     for (int j = 0; j < TAPS; ++j) {
       const int back = TAPS - 1 - j;
@@ -218,14 +222,14 @@ __global__ __launch_bounds__(NT) void short_conv_vec_kernel(const T* __restrict_
 
 template <typename T>
 bool launch_conv_vec(const T* y, int64_t y_stride, int C, const float* w, int taps, const int* ps, const int* ts, const int* qs,
-                     const int* sr, const T* state, int n_rows, T* out, int act, int T_, hipStream_t s) {
+                     const int* sr, const T* state, int n_rows, T* out, int act, int T_, const float* bias, hipStream_t s) {
   constexpr int VEC = 16 / sizeof(T);
   const uintptr_t bits = reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(state) | reinterpret_cast<uintptr_t>(out);
   if (C % VEC || y_stride % VEC || bits % 16 || taps < 2 || taps > 4) return false;
   dim3 grid((T_ + CONV_ROWS - 1) / CONV_ROWS, (C / VEC + NT - 1) / NT);
-  if (taps == 2) short_conv_vec_kernel<T, VEC, 2><<<grid, NT, 0, s>>>(y, y_stride, C, w, ps, ts, qs, sr, state, n_rows, out, act, T_);
-  else if (taps == 3) short_conv_vec_kernel<T, VEC, 3><<<grid, NT, 0, s>>>(y, y_stride, C, w, ps, ts, qs, sr, state, n_rows, out, act, T_);
-  else short_conv_vec_kernel<T, VEC, 4><<<grid, NT, 0, s>>>(y, y_stride, C, w, ps, ts, qs, sr, state, n_rows, out, act, T_);
+  if (taps == 2) short_conv_vec_kernel<T, VEC, 2><<<grid, NT, 0, s>>>(y, y_stride, C, w, ps, ts, qs, sr, state, n_rows, out, act, T_, bias);
+  else if (taps == 3) short_conv_vec_kernel<T, VEC, 3><<<grid, NT, 0, s>>>(y, y_stride, C, w, ps, ts, qs, sr, state, n_rows, out, act, T_, bias);
+  else short_conv_vec_kernel<T, VEC, 4><<<grid, NT, 0, s>>>(y, y_stride, C, w, ps, ts, qs, sr, state, n_rows, out, act, T_, bias);
   return true;
 }
 
@@ -378,10 +382,12 @@ __global__ __launch_bounds__(NT) void hgrn2_prepare_kernel(const T* __restrict__
 
 // Gated delta rule.  One block per token: q / k heads (G of them, from the convolved row c) become
 // unit vectors x / sqrt(sum x^2 + 1e-6), q also times dim^-1/2; beta = sigmoid(y[off_beta + h]);
-// decay g[h, i] = exp(-exp(a_log[h]) softplus(a[h, i] + dt_bias[h, i])).
+// decay g[h, i] = exp(-exp(a_log[h]) softplus(a[h, i] + dt_bias[h, i])), i < gd: gd = dim (a decay per
+// key channel) or 1 (one per head); a rows have their own stride.
 template <typename T>
 __global__ __launch_bounds__(NT) void delta_prepare_kernel(const T* __restrict__ c, int64_t c_stride, const T* __restrict__ y,
                                                            int64_t y_stride, int off_beta, const T* __restrict__ a,
+                                                           int64_t a_stride, int gd,
                                                            const float* __restrict__ a_log, const float* __restrict__ dt_bias,
                                                            float* __restrict__ q32, float* __restrict__ k32,
                                                            float* __restrict__ g32, float* __restrict__ beta, int H, int G,
@@ -400,18 +406,19 @@ __global__ __launch_bounds__(NT) void delta_prepare_kernel(const T* __restrict__
     float* o = (v < G ? q32 : k32) + (static_cast<size_t>(t) * G + (v < G ? v : v - G)) * dim;
     for (int i = lane; i < dim; i += 64) o[i] = Elem<T>::ld(x[i]) * r;
   }
-  const int n = H * dim;
+  const int n = H * gd;
   for (int i = threadIdx.x; i < n; i += NT) {
-    const float z = Elem<T>::ld(a[static_cast<size_t>(t) * n + i]) + dt_bias[i];
+    const float z = Elem<T>::ld(a[static_cast<size_t>(t) * a_stride + i]) + dt_bias[i];
     const float sp = z > 20.f ? z : log1pf(expf(z));
-    g32[static_cast<size_t>(t) * n + i] = expf(-expf(a_log[i / dim]) * sp);
+    g32[static_cast<size_t>(t) * n + i] = expf(-expf(a_log[i / gd]) * sp);
   }
   if (threadIdx.x < H) beta[static_cast<size_t>(t) * H + threadIdx.x] = sigmoidf_(Elem<T>::ld(y[static_cast<size_t>(t) * y_stride + off_beta + threadIdx.x]));
 }
 
 // ---------------------------------------------------------------- the recurrence
 // Per head a dim x vdim fp32 state S; token after token
-//     S <- diag(g_t) S;  u = DELTA ? beta_t (v_t - S^T k_t) : v_t;  S <- S + k_t u^T;  o_t = S^T q_t.
+//     S <- diag(g_t) S;  u = DELTA ? beta_t (v_t - S^T k_t) : beta_t v_t;  S <- S + k_t u^T;  o_t = S^T q_t
+// (beta null without DELTA: u = v_t; gd = 1: g_t is one number per head, else one per key channel).
 // One workgroup of SCAN_WAVES waves per (segment, head, 8 SCAN_WAVES value columns); a wave owns 8
 // columns: lane = 8 column + row group, so a lane keeps
 // dim / 8 rows of one column of S in registers and the two sums over rows (S^T k and S^T q) are
@@ -421,13 +428,13 @@ __global__ __launch_bounds__(NT) void delta_prepare_kernel(const T* __restrict__
 // different banks) by the whole workgroup, so a head's vectors are fetched once per 8 SCAN_WAVES
 // columns; the next chunk's loads fly under this chunk's arithmetic.
 struct ScanArgs {
-  const float* q; const float* k; const float* g;   // [T, Gq, dim], [T, Gq, dim], [T, H, dim]
+  const float* q; const float* k; const float* g;   // [T, Gq, dim], [T, Gq, dim], [T, H, gd]
   const void* v; int64_t v_stride;                  // [T, >= H vdim]
   const float* beta;                                // [T, H]
   const int* positions; const int* q_start; const int* state_rows;
   float* state;                                     // [n_rows, H, dim, vdim]
   float* out;                                       // [T, H, vdim]
-  int n_rows, H, Gq, dim, vdim;
+  int n_rows, H, Gq, dim, vdim, gd;
 };
 
 template <int CTRL>
@@ -479,12 +486,13 @@ __global__ __launch_bounds__(64 * SCAN_WAVES) void state_scan_kernel(ScanArgs a)
     src_ok[n] = which < 3 && i < dim;
     const float* p = which == 0 ? a.q + (static_cast<size_t>(t0) * a.Gq + gq) * dim
                    : which == 1 ? a.k + (static_cast<size_t>(t0) * a.Gq + gq) * dim
-                                : a.g + (static_cast<size_t>(t0) * a.H + h) * dim;
-    src[n] = p + (src_ok[n] ? i : 0);
-    step[n] = which < 2 ? static_cast<int64_t>(a.Gq) * dim : static_cast<int64_t>(a.H) * dim;
+                                : a.g + (static_cast<size_t>(t0) * a.H + h) * a.gd;
+    src[n] = p + ((src_ok[n] && (which < 2 || a.gd > 1)) ? i : 0);
+    step[n] = which < 2 ? static_cast<int64_t>(a.Gq) * dim : static_cast<int64_t>(a.H) * a.gd;
   }
   const T* vsrc = vbase + static_cast<size_t>(t0) * a.v_stride;
-  const float* bsrc = DELTA ? a.beta + static_cast<size_t>(t0) * a.H + h : nullptr;
+  const bool scaled = a.beta != nullptr;   // (always with DELTA)
+  const float* bsrc = scaled ? a.beta + static_cast<size_t>(t0) * a.H + h : nullptr;
   auto load = [&](int first, Chunk& c) {
 #pragma unroll
     for (int tt = 0; tt < CT; ++tt) {
@@ -497,7 +505,7 @@ __global__ __launch_bounds__(64 * SCAN_WAVES) void state_scan_kernel(ScanArgs a)
       c.v[tt] = (live && col_ok) ? Elem<T>::ld(*vsrc) : 0.f;
       vsrc += a.v_stride;
       c.be[tt] = 1.0f;
-      if (DELTA) {
+      if (scaled) {
         if (live) c.be[tt] = *bsrc;
         bsrc += a.H;
       }
@@ -529,6 +537,7 @@ __global__ __launch_bounds__(64 * SCAN_WAVES) void state_scan_kernel(ScanArgs a)
         const f32x4* kv = reinterpret_cast<const f32x4*>(&vec[buf][tt][VP + rg * GP]);
         const f32x4* gv = reinterpret_cast<const f32x4*>(&vec[buf][tt][2 * VP + rg * GP]);
         float u = cur.v[tt];
+        if (!DELTA) u *= cur.be[tt];
         if (DELTA) {
           float d[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -580,11 +589,12 @@ __global__ __launch_bounds__(64 * SCAN_WAVES) void state_scan_kernel(ScanArgs a)
 }
 
 // o fp32 [T, H, vdim] -> out [T, H vdim]: every head over its root mean square, times w [vdim],
-// times sigmoid(gate[t, h vdim + e]) (gate null: none).  One wave per (token, head).
+// times sigmoid(gate[t, h vdim + e]) (gate_kind 0) or silu of it (1) (gate null: none).  One wave per (token, head).
 template <typename T>
 __global__ __launch_bounds__(NT) void head_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ w, float eps,
                                                             const T* __restrict__ gate, int64_t gate_stride,
-                                                            T* __restrict__ out, int64_t n_heads_total, int H, int vdim) {
+                                                            T* __restrict__ out, int64_t n_heads_total, int H, int vdim,
+                                                            int gate_kind) {
   const int lane = threadIdx.x & 63;
   const int64_t th = static_cast<int64_t>(blockIdx.x) * (NT / 64) + (threadIdx.x >> 6);
   if (th >= n_heads_total) return;
@@ -596,7 +606,10 @@ __global__ __launch_bounds__(NT) void head_norm_gate_kernel(const float* __restr
   const int h = static_cast<int>(th - t * H);
   for (int e = lane; e < vdim; e += 64) {
     float v = x[e] * r * w[e];
-    if (gate != nullptr) v *= sigmoidf_(Elem<T>::ld(gate[t * gate_stride + static_cast<int64_t>(h) * vdim + e]));
+    if (gate != nullptr) {
+      const float z = Elem<T>::ld(gate[t * gate_stride + static_cast<int64_t>(h) * vdim + e]);
+      v *= gate_kind == 0 ? sigmoidf_(z) : z * sigmoidf_(z);
+    }
     out[th * vdim + e] = Elem<T>::st(v);
   }
 }
@@ -660,24 +673,24 @@ BCG_API int bcg_residual_mix_norm(void* resid, const void* a, const void* wa, co
 
 BCG_API int bcg_short_conv(const void* y, int64_t y_stride, int C, const void* w, int taps, const void* positions,
                            const void* token_seq, const void* q_start, const void* state_rows, void* state, int n_rows,
-                           void* out, int act, int T_, int B, int is_f32, void* stream) {
+                           void* out, int act, const void* bias, int T_, int B, int is_f32, void* stream) {
   if (T_ <= 0 || C <= 0) return 0;
   if (taps < 1 || taps > MAX_TAPS || (taps > 1 && state == nullptr)) return -2;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int *ps = static_cast<const int*>(positions), *ts = static_cast<const int*>(token_seq),
             *qs = static_cast<const int*>(q_start), *sr = static_cast<const int*>(state_rows);
-  const float* wf = static_cast<const float*>(w);
+  const float *wf = static_cast<const float*>(w), *bf = static_cast<const float*>(bias);
   dim3 grid(T_, (C + NT - 1) / NT), sgrid(B, (C + NT - 1) / NT);
   if (T_ > 2147483647 / 2 || grid.y > 65535) return -2;
   const bool vec = is_f32 ? launch_conv_vec<float>(static_cast<const float*>(y), y_stride, C, wf, taps, ps, ts, qs, sr,
-                                                   static_cast<const float*>(state), n_rows, static_cast<float*>(out), act, T_, s)
+                                                   static_cast<const float*>(state), n_rows, static_cast<float*>(out), act, T_, bf, s)
                           : launch_conv_vec<bf16_t>(static_cast<const bf16_t*>(y), y_stride, C, wf, taps, ps, ts, qs, sr,
-                                                    static_cast<const bf16_t*>(state), n_rows, static_cast<bf16_t*>(out), act, T_, s);
+                                                    static_cast<const bf16_t*>(state), n_rows, static_cast<bf16_t*>(out), act, T_, bf, s);
   if (!vec)
   BCG_BY_TYPE((short_conv_kernel<float><<<grid, NT, 0, s>>>(static_cast<const float*>(y), y_stride, C, wf, taps, ps, ts, qs, sr,
-                                                           static_cast<const float*>(state), n_rows, static_cast<float*>(out), act)),
+                                                           static_cast<const float*>(state), n_rows, static_cast<float*>(out), act, bf)),
               (short_conv_kernel<bf16_t><<<grid, NT, 0, s>>>(static_cast<const bf16_t*>(y), y_stride, C, wf, taps, ps, ts, qs, sr,
-                                                            static_cast<const bf16_t*>(state), n_rows, static_cast<bf16_t*>(out), act)));
+                                                            static_cast<const bf16_t*>(state), n_rows, static_cast<bf16_t*>(out), act, bf)));
   if (taps > 1 && B > 0)
     BCG_BY_TYPE((short_conv_state_kernel<float><<<sgrid, NT, 0, s>>>(static_cast<const float*>(y), y_stride, C, taps, ps, qs, sr,
                                                                     static_cast<float*>(state), n_rows)),
@@ -736,48 +749,48 @@ BCG_API int bcg_hgrn2_prepare(const void* y, int64_t stride, int off_q, int off_
 }
 
 BCG_API int bcg_delta_prepare(const void* c, int64_t c_stride, const void* y, int64_t y_stride, int off_beta, const void* a,
-                              const void* a_log, const void* dt_bias, void* q32, void* k32, void* g32, void* beta, int T_,
-                              int H, int G, int dim, int is_f32, void* stream) {
+                              int64_t a_stride, int gd, const void* a_log, const void* dt_bias, void* q32, void* k32, void* g32,
+                              void* beta, int T_, int H, int G, int dim, int is_f32, void* stream) {
   if (T_ <= 0) return 0;
-  if (H > NT || H <= 0 || G <= 0 || H % G) return -2;
+  if (H > NT || H <= 0 || G <= 0 || H % G || (gd != 1 && gd != dim)) return -2;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const float *al = static_cast<const float*>(a_log), *db = static_cast<const float*>(dt_bias);
   float *q = static_cast<float*>(q32), *k = static_cast<float*>(k32), *g = static_cast<float*>(g32), *be = static_cast<float*>(beta);
   BCG_BY_TYPE((delta_prepare_kernel<float><<<T_, NT, 0, s>>>(static_cast<const float*>(c), c_stride, static_cast<const float*>(y),
-                                                            y_stride, off_beta, static_cast<const float*>(a), al, db, q, k, g, be, H, G, dim)),
+                                                            y_stride, off_beta, static_cast<const float*>(a), a_stride, gd, al, db, q, k, g, be, H, G, dim)),
               (delta_prepare_kernel<bf16_t><<<T_, NT, 0, s>>>(static_cast<const bf16_t*>(c), c_stride, static_cast<const bf16_t*>(y),
-                                                             y_stride, off_beta, static_cast<const bf16_t*>(a), al, db, q, k, g, be, H, G, dim)));
+                                                             y_stride, off_beta, static_cast<const bf16_t*>(a), a_stride, gd, al, db, q, k, g, be, H, G, dim)));
   return BCG_CHECK_LAUNCH();
 }
 
 BCG_API int bcg_gated_state_scan(const void* q32, const void* k32, const void* g32, const void* v, int64_t v_stride,
                                  const void* beta, const void* positions, const void* q_start, const void* state_rows,
-                                 void* state, int n_rows, void* out, int B, int H, int Gq, int dim, int vdim, int delta,
+                                 void* state, int n_rows, void* out, int B, int H, int Gq, int dim, int vdim, int gd, int delta,
                                  int is_f32, void* stream) {
   if (B <= 0) return 0;
-  if (dim < 1 || dim > 256 || H <= 0 || Gq <= 0 || H % Gq || H > 65535 || (delta && beta == nullptr)) return -2;
+  if (dim < 1 || dim > 256 || H <= 0 || Gq <= 0 || H % Gq || H > 65535 || (delta && beta == nullptr) || (gd != 1 && gd != dim)) return -2;
   ScanArgs a;
   a.q = static_cast<const float*>(q32); a.k = static_cast<const float*>(k32); a.g = static_cast<const float*>(g32);
   a.v = v; a.v_stride = v_stride; a.beta = static_cast<const float*>(beta);
   a.positions = static_cast<const int*>(positions); a.q_start = static_cast<const int*>(q_start);
   a.state_rows = static_cast<const int*>(state_rows);
   a.state = static_cast<float*>(state); a.out = static_cast<float*>(out);
-  a.n_rows = n_rows; a.H = H; a.Gq = Gq; a.dim = dim; a.vdim = vdim;
+  a.n_rows = n_rows; a.H = H; a.Gq = Gq; a.dim = dim; a.vdim = vdim; a.gd = gd;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (delta) return is_f32 ? launch_scan<float, true>(a, B, s) : launch_scan<bf16_t, true>(a, B, s);
   return is_f32 ? launch_scan<float, false>(a, B, s) : launch_scan<bf16_t, false>(a, B, s);
 }
 
 BCG_API int bcg_head_norm_gate(const void* o32, const void* w, float eps, const void* gate, int64_t gate_stride, void* out,
-                               int T_, int H, int vdim, int is_f32, void* stream) {
+                               int T_, int H, int vdim, int gate_kind, int is_f32, void* stream) {
   if (T_ <= 0 || H <= 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int64_t n = static_cast<int64_t>(T_) * H;
   const int grid = static_cast<int>((n + NT / 64 - 1) / (NT / 64));
   const float *o = static_cast<const float*>(o32), *wf = static_cast<const float*>(w);
   BCG_BY_TYPE((head_norm_gate_kernel<float><<<grid, NT, 0, s>>>(o, wf, eps, static_cast<const float*>(gate), gate_stride,
-                                                               static_cast<float*>(out), n, H, vdim)),
+                                                               static_cast<float*>(out), n, H, vdim, gate_kind)),
               (head_norm_gate_kernel<bf16_t><<<grid, NT, 0, s>>>(o, wf, eps, static_cast<const bf16_t*>(gate), gate_stride,
-                                                                static_cast<bf16_t*>(out), n, H, vdim)));
+                                                                static_cast<bf16_t*>(out), n, H, vdim, gate_kind)));
   return BCG_CHECK_LAUNCH();
 }
