@@ -203,6 +203,15 @@ def seqmix_ops(lib, linear):
                                  _act(h), _stream()), "moe_route")
         return idx, wts, gate
 
+    def moe_pair_rows(gate, up):
+        """The [2 ff, W] weight of one gated expert as `moe_experts` (kind "silu_gated") reads it:
+        gate and up rows in alternating groups of 16 when ff is a multiple of 16 (the product's
+        epilogue then forms silu(gate) * up), else [gate; up]."""
+        ff, W = gate.shape
+        if ff % 16:
+            return torch.cat([gate, up])
+        return torch.stack([gate.reshape(ff // 16, 16, W), up.reshape(ff // 16, 16, W)], 1).reshape(2 * ff, W)
+
     def moe_experts(h, up, down, idx, weights, kind="relu2"):
         T, W = h.shape
         E, n_up, _ = up.shape
@@ -222,7 +231,11 @@ def seqmix_ops(lib, linear):
         sorted_ = torch.empty(cap, dtype=torch.int32, device=dev)
         tile_e = torch.empty(n_tiles, dtype=torch.int32, device=dev)
         _check(lib.bcg_moe_align(_p(idx), n_slots, E, _p(sorted_), cap, _p(tile_e), n_tiles, _stream()), "moe_align")
-        if gated:   # the stacked projection, then silu(gate) * up over its halves
+        if gated and ff % 16 == 0:   # rows paired by `moe_pair_rows`: silu(gate) * up in the product's epilogue
+            hidden = torch.empty(cap, ff, dtype=h.dtype, device=dev)
+            _check(lib.bcg_moe_gemm(_p(h), W, _p(up), _p(hidden), ff, _p(sorted_), _p(tile_e), n_tiles, n_up, W, top, 1, 0, 2,
+                                    f32, _stream()), "moe gate / up")
+        elif gated:   # the stacked projection, then silu(gate) * up over its halves
             both = torch.empty(cap, n_up, dtype=h.dtype, device=dev)
             _check(lib.bcg_moe_gemm(_p(h), W, _p(up), _p(both), n_up, _p(sorted_), _p(tile_e), n_tiles, n_up, W, top, 1, 0, 0,
                                     f32, _stream()), "moe gate / up")
@@ -242,4 +255,5 @@ def seqmix_ops(lib, linear):
     return dict(embed_scale_rmsnorm=embed_scale_rmsnorm, residual_add_rmsnorm32=residual_add_rmsnorm32,
                 rmsnorm32=rmsnorm32, act_fn=act_fn, rope_multi_kv_write=rope_multi_kv_write,
                 kv_from_logical=kv_from_logical, kv_to_logical=kv_to_logical,
-                multimap_attention=multimap_attention, multimap_tile_rows=multimap_tile_rows, moe_route=moe_route, moe_experts=moe_experts)
+                multimap_attention=multimap_attention, multimap_tile_rows=multimap_tile_rows, moe_route=moe_route, moe_experts=moe_experts,
+                moe_pair_rows=moe_pair_rows)

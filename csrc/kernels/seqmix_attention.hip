@@ -431,10 +431,10 @@ int launch_prefill(const AttnArgs& a, int n_tiles, int tile_rows, hipStream_t s)
   if constexpr (sizeof(T) == 2) if (full && a.maps == 1 && a.swz && a.BS == 16) {   // one-map heads, exact shapes
 #define BCG_EXACT1(KC_, VT_)                                                                     \
   if (a.dim == 16 * KC_ && a.vdim == 16 * VT_) {                                                 \
-    prefill_kernel<T, KC_, VT_, 2, true, true, 2, 1><<<grid, 256, 0, s>>>(a);                    \
+    prefill_kernel<T, KC_, VT_, 2, true, true, 2, 1, 1><<<grid, 256, 0, s>>>(a);                 \
     return BCG_CHECK_LAUNCH();                                                                   \
   }
-    BCG_EXACT1(8, 8) BCG_EXACT1(4, 4) BCG_EXACT1(4, 8) BCG_EXACT1(2, 2) BCG_EXACT1(6, 6)
+    BCG_EXACT1(8, 8) BCG_EXACT1(4, 4) BCG_EXACT1(4, 8) BCG_EXACT1(2, 2) BCG_EXACT1(6, 6) BCG_EXACT1(6, 4) BCG_EXACT1(12, 8)
 #undef BCG_EXACT1
   }
   if constexpr (sizeof(T) == 2) if (small) {
@@ -471,9 +471,9 @@ int launch_decode(const AttnArgs& a, int n_items, hipStream_t s) {
 #define BCG_EXACT1(KC_, VT_)                                                                     \
   if (!done && a.dim == 16 * KC_ && a.vdim == 16 * VT_) {                                        \
     done = true;                                                                                 \
-    decode_mfma_kernel<T, KC_, VT_, 2, true, true, 2, 1><<<grid, 64, 0, s>>>(a);                 \
+    decode_mfma_kernel<T, KC_, VT_, 2, true, true, 2, 1, 1><<<grid, 64, 0, s>>>(a);              \
   }
-    BCG_EXACT1(8, 8) BCG_EXACT1(4, 4) BCG_EXACT1(4, 8) BCG_EXACT1(2, 2) BCG_EXACT1(6, 6)
+    BCG_EXACT1(8, 8) BCG_EXACT1(4, 4) BCG_EXACT1(4, 8) BCG_EXACT1(2, 2) BCG_EXACT1(6, 6) BCG_EXACT1(6, 4) BCG_EXACT1(12, 8)
 #undef BCG_EXACT1
   }
   if constexpr (sizeof(T) == 2) if (!done && a.dim <= 64 && a.vdim <= 128) {

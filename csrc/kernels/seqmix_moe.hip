@@ -94,8 +94,33 @@ __global__ __launch_bounds__(1024) void align_kernel(const int* __restrict__ idx
   }
 }
 
+// Epilogue of a gated expert's first product (act 2).  The N rows of the expert's weight are its
+// gate and up rows in alternating groups of 16 ([gate 0..15 | up 0..15 | gate 16..31 | ...]), so a
+// wave's n tiles 0 / 2 hold gate columns and tiles 1 / 3 the up columns of the SAME features:
+// out[r, f] = silu(gate_f) * up_f with f = n / 2 (N / 2 output columns), both factors and the
+// activation rounded to T like a projection's output.
+template <typename T>
+__device__ __forceinline__ void store_gated(const f32x4 (&acc)[4][4], const int (&slot)[4], T* __restrict__ out,
+                                            int64_t out_stride, int scatter, int p0, int n0, int N, int col, int grp) {
+  auto rnd = [](float v) { return Elem<T>::ld(Elem<T>::st(v)); };
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    if (slot[j] < 0) continue;
+    const int64_t r = scatter ? slot[j] : p0 + 16 * j + col;
+#pragma unroll
+    for (int i2 = 0; i2 < 2; ++i2)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        if (n0 + 32 * i2 + 16 + 4 * grp + q < N) {
+          const float g = rnd(acc[2 * i2][j][q]), u = rnd(acc[2 * i2 + 1][j][q]);
+          out[r * out_stride + (n0 >> 1) + 16 * i2 + 4 * grp + q] = Elem<T>::st(rnd(g / (1.0f + expf(-g))) * u);
+        }
+      }
+  }
+}
+
 // Position p of tile blockIdx.x: slot = sorted[p] (-1: padding).  gather: A row = a[(slot / top)]
-// (token rows), else a[p].  scatter: output row = slot, else p.  act 1: relu squared.
+// (token rows), else a[p].  scatter: output row = slot, else p.  act 1: relu squared; act 2: `store_gated`.
 template <typename T, bool FULL>
 __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ a, int64_t a_stride, const T* __restrict__ w,
                                                        T* __restrict__ out, int64_t out_stride,
@@ -141,6 +166,10 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ a, 
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j) acc[i][j] = mma16(wf[i], af[j], acc[i][j]);
+  }
+  if (act == 2) {
+    store_gated<T>(acc, slot, out, out_stride, scatter, p0, n0, N, col, grp);
+    return;
   }
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
@@ -253,6 +282,10 @@ __global__ __launch_bounds__(256) void moe_gemm_lds_kernel(const T* __restrict__
     }
   }
   const int n0 = nb + 64 * wave;
+  if (act == 2) {
+    store_gated<T>(acc, slot, out, out_stride, scatter, p0, n0, N, col, grp);
+    return;
+  }
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     if (slot[j] < 0) continue;
@@ -317,7 +350,7 @@ BCG_API int bcg_moe_gemm(const void* a, int64_t a_stride, const void* w, void* o
                          const void* tile_expert, int n_tiles, int N, int K, int top, int gather, int scatter, int act,
                          int is_f32, void* stream) {
   if (n_tiles <= 0) return 0;
-  if (N < 1 || K < 1 || n_tiles > (1 << 24) || (N + TN - 1) / TN > 65535) return -2;
+  if (N < 1 || K < 1 || n_tiles > (1 << 24) || (N + TN - 1) / TN > 65535 || (act == 2 && N % 32)) return -2;
   hipStream_t s = static_cast<hipStream_t>(stream);
   dim3 grid(n_tiles, (N + TN - 1) / TN);
   const int vec = (K % 4 == 0 && a_stride % 4 == 0) ? 1 : 0;

@@ -1,0 +1,316 @@
+"""Checks of the Mabivik mechanisms and engine schedules against the float64 oracle, written once
+for both backends: ``Env("torch", "cpu", ...)`` runs the PyTorch reference ops, ``Env("hip", "cuda",
+...)`` the HIP kernels.  Every mixer is driven alone, over shuffled pages and state rows, whole and
+in portions, with an input of the test's making."""
+import numpy as np
+import torch
+
+import mabivik_cases as C
+import mabivik_oracle as O
+from byzantine_consensus_llm_agents_amd.models.config import MabivikConfig
+from byzantine_consensus_llm_agents_amd.models.mabivik import MabivikModel
+from byzantine_consensus_llm_agents_amd.ops import get_ops
+
+
+class Env:
+    def __init__(self, backend, device, dtype=torch.float32):
+        self.backend, self.device, self.dtype = backend, device, dtype
+        self.ops = get_ops(backend)
+
+    def close(self, got, want, tol=None):
+        got, want = got.detach().double().cpu().numpy(), np.asarray(want)
+        if self.dtype == torch.float32:
+            tol = tol or 2e-3
+            np.testing.assert_allclose(got, want, atol=tol, rtol=tol)
+        else:   # bf16 activations: error relative to the spread of the expected values
+            err = np.sqrt(((got - want) ** 2).mean(-1)) / max(float(want.std()), 1e-6)
+            assert float(err.max()) < 0.1, float(err.max())
+            assert float(np.median(err)) < 0.04, float(np.median(err))
+
+    def t(self, x, dtype=None):
+        return torch.as_tensor(np.asarray(x)).to(device=self.device, dtype=dtype or self.dtype, copy=True)
+
+
+def rand_bf16(g, *shape, scale=1.0):
+    return (torch.randn(*shape, generator=g) * scale).to(torch.bfloat16).float()
+
+
+# ------------------------------------------------------------------ norms around the stream
+def check_norms(env):
+    g = torch.Generator().manual_seed(0)
+    T, W = 7, 44
+    x0, y = rand_bf16(g, T, W, scale=3.0), rand_bf16(g, T, W, scale=2.0)
+    w1, b1, w2, b2, wr = (rand_bf16(g, W) for _ in range(5))
+    sd = {"n1": w1.double().numpy(), "n1.b": b1.double().numpy(), "n1.alpha": np.float64(0.7),
+          "n2": w2.double().numpy(), "n2.b": b2.double().numpy(), "n2.alpha": np.float64(-0.4)}
+    f = lambda a: env.t(a, torch.float32)  # noqa: E731
+    x = f(x0)
+    h = env.ops.residual_post_norm(x, env.t(y), ("dyt", 0.7, f(w1), f(b1)), ("dyt", -0.4, f(w2), f(b2)), env.dtype)
+    want_x = x0.double().numpy() + O.dyt(sd, "n1", y.double().numpy())
+    env.close(x, want_x, 1e-5) if env.dtype == torch.float32 else env.close(x, want_x)
+    env.close(h, O.dyt(sd, "n2", want_x), 1e-5)
+    # RMS post norm of an fp32 sublayer output, then a rounded copy of the stream
+    y2 = rand_bf16(g, T, W)
+    h2 = env.ops.residual_post_norm(x, f(y2), ("rms", f(wr), 1e-5), ("copy",), env.dtype)
+    want_x2 = want_x + O.unit_rms(y2.double().numpy(), 1e-5) * wr.double().numpy()
+    env.close(x, want_x2, 1e-5) if env.dtype == torch.float32 else env.close(x, want_x2)
+    env.close(h2, want_x2, 1e-5)
+    assert env.ops.residual_post_norm(x, env.t(y), ("dyt", 0.7, f(w1), f(b1)), None, env.dtype) is None
+    # embedding
+    table = rand_bf16(g, 11, W)
+    toks = torch.tensor([3, 0, 10, 3], dtype=torch.int32, device=env.device)
+    xe, he = env.ops.embed_scale_dyt(toks, env.t(table), 2.5, (0.7, f(w1), f(b1)), env.dtype)
+    want = table.double().numpy()[[3, 0, 10, 3]] * 2.5
+    env.close(xe, want, 1e-5)
+    env.close(he, O.dyt(sd, "n1", want), 1e-5)
+
+
+def check_conv_bias(env, taps, cuts):
+    g = torch.Generator().manual_seed(taps)
+    n, ch = sum(cuts), 20
+    y = rand_bf16(g, n, ch + 5)
+    w, b = rand_bf16(g, ch, taps, scale=0.5), rand_bf16(g, ch, scale=0.5)
+    want = O.silu(O.short_conv(y[:, 3:3 + ch].double().numpy(), w.double().numpy(), b.double().numpy()))
+    state = torch.full((3, max(taps - 1, 0), ch), 9.0).to(device=env.device, dtype=env.dtype)   # stale rows
+    at, outs = 0, []
+    for c in cuts:
+        meta = C.segments([(at, c)], [1], env.device)
+        outs.append(env.ops.short_conv(env.t(y[at:at + c])[:, 3:], ch, env.t(w, torch.float32), meta, state, "silu",
+                                       env.t(b, torch.float32)))
+        at += c
+    env.close(torch.cat(outs), want)
+
+
+# ------------------------------------------------------------------ one mixer alone
+def _one_layer(env, layers, width, seed):
+    cfg_dict = C.config(layers, width=width, vocab=29, side=0)
+    cfg = MabivikConfig.from_dict(cfg_dict, "t")
+    model = MabivikModel(cfg, env.ops, env.device, env.dtype)
+    sd = model.random_state_dict(seed, std=0.2)
+    return cfg, model, sd
+
+
+def run_mixer(env, layers, T, cuts=None, craft=None, seed=0, width=40, lens=None):
+    """Drive the LAST layer's mixer alone over the portions ``cuts`` of one sequence (earlier
+    latent layers only write their cache, from inputs of their own).  ``craft(sd, hs)`` may edit
+    the weights and the per-layer inputs.  Returns (got [T, W], want [T, W])."""
+    cfg, model, sd = _one_layer(env, layers, width, seed)
+    g = torch.Generator().manual_seed(seed + 100)
+    hs = [rand_bf16(g, T, width) for _ in layers]
+    if craft:
+        craft(sd, hs)
+    model.load_hf_state_dict(sd)
+    sd64 = O.to_f64(sd)
+    eps = cfg.rms_eps
+    last = len(layers) - 1
+    spec = layers[last]
+    p = f"l{last}.mix."
+    h64 = hs[last].double().numpy()
+    if spec["type"] == "latent_attention":
+        src = spec["mixer"].get("kv_from")
+        j = last if src is None else src
+        kv = O.latent_kv(sd64, f"l{j}.mix.", layers[j]["mixer"], hs[j].double().numpy(), eps)
+        want = O.latent_attention(sd64, p, spec["mixer"], h64, eps, kv)
+    elif spec["type"] == "delta":
+        want = O.delta_mixer(sd64, p, spec["mixer"], h64, eps)
+    else:
+        want = O.mamba2_mixer(sd64, p, spec["mixer"], h64, eps)
+    pages = C.Pages([T, 5, T], seed=seed, device=env.device)   # sequence 2 is ours: state row 2
+    ks, vs = model.alloc_kv(pages.num_blocks, 16, env.dtype)
+    state = model.alloc_state(4)
+    for L in state["layers"]:
+        if L is not None:   # stale state of an earlier owner
+            L["S"].fill_(3.0)
+            if L["conv"] is not None:
+                L["conv"].fill_(-2.0)
+    at, outs = 0, []
+    for c in cuts or [T]:
+        meta = pages.meta([(2, at, c)])
+        meta.state = state
+        for i, l in enumerate(layers):
+            m, L = model.cfg.layers[i].mixer, model.layers[i]
+            h = env.t(hs[i][at:at + c])
+            if l["type"] == "latent_attention":
+                if i == last:
+                    outs.append(model._latent_attention(m, L, h, meta, ks[i], vs[i], None))
+                elif m.kv_from < 0:
+                    model._latent_attention(m, L, h, meta, ks[i], vs[i], None)
+            elif i == last and l["type"] == "delta":
+                outs.append(model._delta(m, L, state["layers"][i], h, meta, None))
+            elif i == last:
+                outs.append(model._mamba2(m, L, state["layers"][i], h, meta, None))
+        at += c
+    return torch.cat(outs), want
+
+
+def loud_key(pos, factor=40.0):
+    """Input row ``pos`` scaled up: its rotated key part (which no norm touches) dominates the scores
+    of about half of the later (query, head) pairs, so dropping or adding that key shows."""
+    def craft(sd, hs):
+        for h in hs:
+            h[pos] *= factor
+    return craft
+
+
+def check_window_edge(env, window=9, T=30, loud=5, cuts=None):
+    m = C.latent(2, 16, 8, 16, 12, 16, window, 10000.0, None)
+    got, want = run_mixer(env, [C.layer("latent_attention", m, 0)], T, cuts, loud_key(loud), seed=5)
+    env.close(got, want)
+    inside, outside = want[loud + window - 1], want[loud + window]
+    assert np.abs(inside - outside).max() > 0.05   # the edge is visible far above the tolerance
+    return got
+
+
+# ------------------------------------------------------------------ feed-forward, token input
+def check_experts(env, E, top, ff, W=40, T=23):
+    g = torch.Generator().manual_seed(E * 10 + top)
+    vocab = 17
+    sd = {}
+    for e in range(E):
+        sd[f"e{e}.gate"], sd[f"e{e}.up"], sd[f"e{e}.down"] = rand_bf16(g, ff, W, scale=0.3), rand_bf16(g, ff, W, scale=0.3), rand_bf16(g, W, ff, scale=0.3)
+    table = torch.stack([torch.randperm(E, generator=g)[:top] for _ in range(vocab)]).to(torch.int32)
+    sd["table"] = table
+    h = rand_bf16(g, T, W)
+    toks = torch.randint(0, vocab, (T,), generator=g).to(torch.int32)
+    want = O.table_experts(O.to_f64(sd), "", {"router": {"top": top}}, h.double().numpy(), toks.tolist())
+    pair = getattr(env.ops, "moe_pair_rows", None)
+    up = torch.stack([(pair(env.t(sd[f"e{e}.gate"]), env.t(sd[f"e{e}.up"])) if pair else torch.cat([env.t(sd[f"e{e}.gate"]), env.t(sd[f"e{e}.up"])]))
+                      for e in range(E)]).contiguous()
+    down = torch.stack([env.t(sd[f"e{e}.down"]) for e in range(E)]).contiguous()
+    idx, wts = env.ops.moe_table_route(toks.to(env.device), table.to(env.device), top)
+    assert idx.cpu().tolist() == table[toks.long()].tolist() and abs(float(wts.min()) - 1.0 / top) < 1e-7
+    env.close(env.ops.moe_experts(env.t(h), up, down, idx, wts, "silu_gated"), want)
+
+
+def check_token_side(env):
+    g = torch.Generator().manual_seed(3)
+    T, W, dim, n_layers = 9, 36, 5, 3
+    cfg = {"token_side": {"dim": dim}}
+    sd = {"side.embed": rand_bf16(g, 13, n_layers * dim), "l1.side.gate": rand_bf16(g, dim, W, scale=0.3),
+          "l1.side.proj": rand_bf16(g, W, dim), "l1.side.norm": rand_bf16(g, W)}
+    x0 = rand_bf16(g, T, W, scale=2.0)
+    toks = torch.randint(0, 13, (T,), generator=g).to(torch.int32)
+    want = x0.double().numpy() + O.token_side(O.to_f64(sd), cfg, 1, x0.double().numpy(), toks.tolist(), 1e-5)
+    x = env.t(x0, torch.float32)
+    z = env.ops.gelu_gather_mul(env.ops.linear(env.t(x0), env.t(sd["l1.side.gate"])), toks.to(env.device), env.t(sd["side.embed"]), dim)
+    env.ops.residual_post_norm(x, env.ops.linear(z, env.t(sd["l1.side.proj"])), ("rms", env.t(sd["l1.side.norm"], torch.float32), 1e-5),
+                               None, env.dtype)
+    env.close(x, want)
+
+
+# ------------------------------------------------------------------ engine schedules
+def whole_prompt(env, cfg, sd, eng, n=45):
+    toks = C.tokens(n, cfg["vocab"], 1)
+    env.close(eng.stream_step([("a", toks, list(range(n)))], end=["a"]), O.forward(sd, cfg, toks))
+
+
+def stream_after_every_layer(env, cfg, sd, eng):
+    toks = C.tokens(19, cfg["vocab"], 2)
+    want = []
+    O.forward(sd, cfg, toks, want)
+    pages = C.Pages([19], device=env.device)
+    meta = pages.meta([(0, 0, 19)])
+    meta.state = eng.model.alloc_state(2)
+    k, v = eng.model.alloc_kv(pages.num_blocks, 16, env.dtype)
+    got = []
+    eng.model.forward(torch.tensor(toks, dtype=torch.int32, device=env.device), meta, k, v, trace=got)
+    assert len(got) == len(want) == len(cfg["layers"])
+    for a, b in zip(got, want):
+        env.close(a, b)
+
+
+def prefill_then_token_by_token(env, cfg, sd, eng, n=70, first=30):
+    toks = C.tokens(n, cfg["vocab"], 3)
+    want = O.forward(sd, cfg, toks)
+    env.close(eng.stream_step([("d", toks[:first], [0, 1, first - 1])]), want[[0, 1, first - 1]])
+    got = [eng.stream_step([("d", toks[p:p + 1], [0])], end=["d"] if p == n - 1 else []) for p in range(first, n)]
+    env.close(torch.cat(got), want[first:])   # crosses page borders and every window's edge
+
+
+def first_tokens_one_by_one(env, cfg, sd, eng):
+    toks = C.tokens(7, cfg["vocab"], 4)
+    want = O.forward(sd, cfg, toks)
+    got = [eng.stream_step([("f", toks[p:p + 1], [0])], end=["f"] if p == 6 else []) for p in range(7)]
+    env.close(torch.cat(got), want)
+
+
+def portions(env, cfg, sd, eng, sizes):
+    n = sum(sizes)
+    toks = C.tokens(n, cfg["vocab"], 5)
+    want = O.forward(sd, cfg, toks)
+    at, got = 0, []
+    for i, s in enumerate(sizes):
+        got.append(eng.stream_step([("p", toks[at:at + s], list(range(s)))], end=["p"] if i == len(sizes) - 1 else []))
+        at += s
+    env.close(torch.cat(got), want)
+
+
+def mixed_batches_and_reuse(env, cfg, sd, eng, lens=(70, 33, 18, 64, 41, 90, 5, 36)):
+    """Up to four live requests, portions beside single tokens, rows sitting out; twice as many
+    requests as state rows over a pool smaller than the work: pages and rows are used again."""
+    reqs = {f"r{i}": C.tokens(n, cfg["vocab"], 10 + i) for i, n in enumerate(lens)}
+    want = {k: O.forward(sd, cfg, t) for k, t in reqs.items()}
+    at = {k: 0 for k in reqs}
+    waiting, live, step = list(reqs), [], 0
+    free_at_start = eng.blocks.num_free_blocks
+    got, expect = [], []
+    while waiting or live:
+        while waiting and len(live) < 4:
+            live.append(waiting.pop(0))
+        entries, end = [], []
+        for j, k in enumerate(live):
+            if (step + j) % 5 == 4 and at[k] > 0:
+                continue
+            take = [1, 2, 16, 7, 1, 19][(step + j) % 6] if at[k] > 0 else [20, 3, 16][j % 3]
+            take = min(take, len(reqs[k]) - at[k])
+            entries.append((k, reqs[k][at[k]:at[k] + take], list(range(take))))
+            expect.append(want[k][at[k]:at[k] + take])
+            at[k] += take
+            if at[k] == len(reqs[k]):
+                end.append(k)
+        if entries:
+            got.append(eng.stream_step(entries, end))
+        live = [k for k in live if k not in end]
+        step += 1
+    env.close(torch.cat(got), np.concatenate(expect))
+    assert eng.blocks.num_free_blocks == free_at_start and not any(eng.slots)
+    assert sum(lens) > 16 * free_at_start / 2
+
+
+def greedy_generation(env, cfg, sd, eng, tie=1e-3):
+    prompts = [C.tokens(n, cfg["vocab"], 20 + n) for n in (9, 31, 16, 2, 40, 23)]
+    budgets = (6, 4, 17, 5, 3, 11)
+    outs = eng.generate_ids(prompts, max_tokens=list(budgets), temperature=0.0)
+    for p, out, n in zip(prompts, outs, budgets):
+        assert len(out) == n
+        seq = list(p)
+        for tok in out:
+            logits = O.forward(sd, cfg, seq)[-1]
+            top2 = np.sort(logits)[-2:]
+            if float(top2[1] - top2[0]) < tie * max(1.0, float(logits.std())):
+                break  # a near tie: either token is a correct greedy step
+            assert tok == int(logits.argmax())
+            seq.append(tok)
+
+
+def drawn_configuration(env, tmp_path, seed, pool_tokens=256):
+    cfg = C.random_config(seed)
+    path = str(tmp_path / "m")
+    sd = O.to_f64(C.checkpoint(cfg, path, seed=seed))
+    eng = C.engine(path, backend=env.backend, dtype=env.dtype, pool_tokens=pool_tokens)
+    try:
+        a, b = C.tokens(60, cfg["vocab"], seed), C.tokens(23, cfg["vocab"], seed + 100)
+        wa, wb = O.forward(sd, cfg, a), O.forward(sd, cfg, b)
+        env.close(eng.stream_step([("w", a, list(range(60)))], end=["w"]), wa)
+        at, got, want = 0, [], []
+        for i, s in enumerate([3, 2, 30, 1, 1, 17, 2, 4]):
+            entries = [("a", a[at:at + s], list(range(s))), ("b", b[i:i + 1], [0])]
+            want += [wa[at:at + s], wb[i:i + 1]]
+            at += s
+            got.append(eng.stream_step(entries))
+        env.close(torch.cat(got), np.concatenate(want))
+        assert at == 60
+        eng.stream_step([("b", b[8:], [])], end=["a", "b"])
+        assert not any(eng.slots)
+    finally:
+        eng.shutdown()
