@@ -122,7 +122,7 @@ def parse(argv=None):
                          "all-reduce kernels forced over IPC peer buffers (never for measurements)")
     ap.add_argument("--verbose", action="store_true")
     ap.add_argument("--family-compare", action="store_true",
-                    help="instead of the headline workload: prefill / decode tokens/s of the Mofidra and Padadra families beside "
+                    help="instead of the headline workload: prefill / decode tokens/s of the Mofidra, Padadra and Mabivik families beside "
                          "the Qwen3-style decoder at equal layer sizes, and their hot kernels against the roofline "
                          "(one GPU, random weights; utils/family_bench.py)")
     return ap.parse_args(argv)

@@ -1,4 +1,4 @@
-"""Prefill / decode throughput of the Mofidra and Padadra families beside the Qwen3-style decoder
+"""Prefill / decode throughput of the Mofidra, Padadra and Mabivik families beside the Qwen3-style decoder
 at equal layer sizes (random weights, synthetic tokens), and the hot kernels against their
 rooflines.  ``bench.py --family-compare`` prints the result as one JSON line.
 
@@ -14,6 +14,16 @@ rule has the query-head count, half as many q / k heads, 128 x 128 state and 4-t
 one layer in four is a delta layer.  Its closest relative is Mofidra (the same fp32 stream,
 parallel sublayers and attention kernels).
 
+Mabivik at equal size: the same width and head count; four layers (latent attention, state
+space, delta rule, a second latent attention that reads the first one's cache); the latent
+attention has 128 unrotated + 64 rotated query / key features and 128 value features per head, a
+768-wide query latent, a 128-wide key / value latent (a cached row of 192 features, ONE KV head for
+all query heads) and a 512-key window; the state-space mixer 2 x width / 128 heads of 128 x 128
+state in two groups; the delta rule the query-head count of 128 x 128 states with one decay per
+head; 4-tap convolutions; every feed-forward routes top-2 of 8 gated experts of ff/4 by the token id
+(Mofidra's MoE variant is its relative there); a 256-wide token input per layer.  Its closest
+relative is Padadra (fp32 stream, windowed attention beside recurrences, the same state tables).
+
 Rooflines: 2.5 PFLOP/s dense bf16 MFMA, 8 TB/s HBM.  A kernel's ``roof_frac`` is
 max(flops / peak, bytes / bandwidth) / measured time.  The recurrence runs on the vector ALUs:
 its compute roof is 157 TFLOP/s fp32.
@@ -24,7 +34,8 @@ import time
 
 import torch
 
-from ..models.config import MofidraConfig, ModelConfig, PadadraConfig
+from ..models.config import MabivikConfig, MofidraConfig, ModelConfig, PadadraConfig
+from ..models.mabivik import MabivikModel
 from ..models.mofidra import MofidraModel
 from ..models.padadra import PadadraModel
 from ..models.transformer import AttnMeta, DecoderModel
@@ -63,6 +74,25 @@ def padadra_config(s) -> PadadraConfig:
     return PadadraConfig.from_dict({"architecture": "Padadra", "width": s["width"], "vocab": s["vocab"],
                                     "embedding": {"scale": 1.0, "bigram": {"buckets": 65521, "mul_prev": 1000003, "mul_cur": 31}},
                                     "norm": {"eps": 1e-5}, "residual_mult": 0.5, "layers": layers}, "padadra-bench")
+
+
+def mabivik_config(s) -> MabivikConfig:
+    H, W = s["heads"], s["width"]
+    rot = {"dims": 64, "base": 1e6, "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}
+    lat = {"heads": H, "dim": 128, "rot_dim": 64, "vdim": 128, "q_rank": 768, "kv_rank": 128, "scale": 0.072, "rot": rot,
+           "mask": {"size": 512}}
+    mlp = {"kind": "moe", "expert": {"ff": s["ff"] // 4}, "router": {"experts": 8, "top": 2}}
+    kinds = [("latent_attention", lat), ("mamba2", {"heads": 2 * W // 128, "vdim": 128, "state": 128, "groups": 2, "norm_groups": 2, "conv": 4}),
+             ("delta", {"heads": H, "kv_heads": H // 2, "dim": 128, "vdim": 128, "conv": 4}), ("latent_attention", dict(lat, kv_from=0))]
+    layers = []
+    for i in range(s["layers"]):
+        kind, mixer = kinds[i % 4]
+        if kind == "latent_attention" and "kv_from" in mixer:
+            mixer = dict(mixer, kv_from=i - 3)
+        layers.append({"type": kind, "mixer": mixer, "mlp": mlp})
+    return MabivikConfig.from_dict({"architecture": "Mabivik", "width": W, "vocab": s["vocab"], "embedding": {"scale": 1.0},
+                                    "norm": {"eps": 1e-5}, "logit_scale": 1.0, "token_side": {"dim": 256}, "layers": layers},
+                                   "mabivik-bench")
 
 
 def decoder_config(s) -> ModelConfig:
@@ -300,6 +330,150 @@ def state_kernels(s, dev):
     return out
 
 
+def latent_kernels(s, dev):
+    """The Mabivik kernels beside their like kernels of Padadra / Mofidra at the same shapes."""
+    ops = get_ops("hip")
+    H, G, W = s["heads"], s["kv_heads"], s["width"]
+    bf = torch.bfloat16
+    out = {}
+    n, ctx, window = 8, 1024, 512
+    T, b = n * ctx, 64
+    R, RD = 128, 64
+    KD = R + RD
+    pairs = sum(min(i + 1, window) for i in range(ctx)) * n
+    meta, nb = step_meta(n, ctx, ctx, 64, dev, True)
+    dmeta, nbd = step_meta(b, ctx, 1, 64, dev, True)
+    nb = max(nb, nbd)
+    # ---- prefill attention, 8 x 1024, 512-key window: one KV head of 192 key / 128 value features against GQA heads of 128 / 128 ----
+    q = torch.randn(T, H, KD, device=dev, dtype=bf)
+    kc, vc = torch.randn(nb, 1, BS, KD, device=dev, dtype=bf), torch.randn(nb, 1, R, BS, device=dev, dtype=bf)
+    t = _time(lambda: ops.multimap_attention(q, kc, vc, meta, 0.072, 1, 0.0, -1.0, 1.0, R, window, None))
+    out["prefill_attention"] = {"mabivik_ms": round(t * 1e3, 3),
+                                "mabivik_roof_frac": _roof(2 * H * (KD + R) * pairs, T * H * (KD + R) * 2 + T * (KD + R) * 2, t)}
+    q1 = torch.randn(T, H, 128, device=dev, dtype=bf)
+    k1, v1 = torch.randn(nb, G, BS, 128, device=dev, dtype=bf), torch.randn(nb, G, 128, BS, device=dev, dtype=bf)
+    sink = torch.randn(H, device=dev)
+    t = _time(lambda: ops.multimap_attention(q1, k1, v1, meta, 0.088, 1, 0.0, -1.0, 1.0, 128, window, sink))
+    out["prefill_attention"].update({"padadra_ms": round(t * 1e3, 3),
+                                     "padadra_roof_frac": _roof(2 * H * 256 * pairs, T * H * 256 * 2 + T * G * 256 * 2, t)})
+    # ---- decode attention, 64 rows x 1024 context ----
+    qd, qd1 = torch.randn(b, H, KD, device=dev, dtype=bf), torch.randn(b, H, 128, device=dev, dtype=bf)
+    t = _graph_time(lambda: ops.multimap_attention(qd, kc, vc, dmeta, 0.072, 1, 0.0, -1.0, 1.0, R, window, None), iters=50)
+    out["decode_attention"] = {"mabivik_ms": round(t * 1e3, 4),
+                               "mabivik_roof_frac": _roof(2 * H * (KD + R) * b * window, b * window * (KD + R) * 2, t)}
+    t = _graph_time(lambda: ops.multimap_attention(qd1, k1, v1, dmeta, 0.088, 1, 0.0, -1.0, 1.0, 128, window, sink), iters=50)
+    out["decode_attention"].update({"padadra_ms": round(t * 1e3, 4),
+                                    "padadra_roof_frac": _roof(2 * H * 256 * b * window, b * window * G * 256 * 2, t)})
+    # ---- decode attention, 512 rows x 1024 context: enough waves to fill the chip with one KV head ----
+    b2 = 512
+    dmeta2, nb2 = step_meta(b2, ctx, 1, 64, dev, True)
+    kc2, vc2 = torch.randn(nb2, 1, BS, KD, device=dev, dtype=bf), torch.randn(nb2, 1, R, BS, device=dev, dtype=bf)
+    k12, v12 = torch.randn(nb2, G, BS, 128, device=dev, dtype=bf), torch.randn(nb2, G, 128, BS, device=dev, dtype=bf)
+    qd2, qd12 = torch.randn(b2, H, KD, device=dev, dtype=bf), torch.randn(b2, H, 128, device=dev, dtype=bf)
+    t = _graph_time(lambda: ops.multimap_attention(qd2, kc2, vc2, dmeta2, 0.072, 1, 0.0, -1.0, 1.0, R, window, None), iters=50)
+    out["decode_attention_512_rows"] = {"mabivik_ms": round(t * 1e3, 4),
+                                        "mabivik_roof_frac": _roof(2 * H * (KD + R) * b2 * window, b2 * window * (KD + R) * 2, t)}
+    t = _graph_time(lambda: ops.multimap_attention(qd12, k12, v12, dmeta2, 0.088, 1, 0.0, -1.0, 1.0, 128, window, sink), iters=50)
+    out["decode_attention_512_rows"].update({"padadra_ms": round(t * 1e3, 4),
+                                             "padadra_roof_frac": _roof(2 * H * 256 * b2 * window, b2 * window * G * 256 * 2, t)})
+    del kc2, vc2, k12, v12
+    # ---- residual update + next norm, 8192 rows: dynamic tanh (no reduction) against the RMS kernels ----
+    x32 = torch.randn(T, W, device=dev)
+    a, c, p = (torch.randn(T, W, device=dev, dtype=bf) for _ in range(3))
+    w1, b1, w2, b2 = (torch.randn(W, device=dev) for _ in range(4))
+    t = _time(lambda: ops.residual_post_norm(x32, a, ("dyt", 0.5, w1, b1), ("dyt", 0.7, w2, b2), bf), iters=20)
+    out["residual_norm"] = {"mabivik_ms": round(t * 1e3, 4), "mabivik_roof_frac": _roof(0, T * W * (4 + 4 + 2 + 2), t)}
+    f32part = torch.randn(T, W, device=dev)
+    t = _time(lambda: ops.residual_post_norm(x32, f32part, ("rms", w1, 1e-5), ("dyt", 0.7, w2, b2), bf), iters=20)
+    out["residual_norm_rms_post"] = {"mabivik_ms": round(t * 1e3, 4), "mabivik_roof_frac": _roof(0, T * W * (4 + 4 + 4 + 2), t)}
+    t = _time(lambda: ops.residual_mix_norm(x32, [(a, w1), (c, w2)], 0.5, [p], 0.5, 1e-5, (1.0, 0.9), bf), iters=20)
+    out["residual_norm"].update({"padadra_ms": round(t * 1e3, 4), "padadra_roof_frac": _roof(0, T * W * (4 + 4 + 3 * 2 + 2 * 2), t)})
+    w32 = torch.zeros(W, device=dev)
+    t = _time(lambda: ops.residual_add_rmsnorm32(x32, [a, p], w32, 1e-5, 1.0, bf), iters=20)
+    out["residual_norm"].update({"mofidra_ms": round(t * 1e3, 4), "mofidra_roof_frac": _roof(0, T * W * (4 + 4 + 2 + 2 + 2), t)})
+    # ---- cache write, 8192 rows: latent norm + rotary + two slab writes against Padadra's q / k / v rotary write ----
+    fused = 768 + KD + H * 128
+    y = torch.randn(T, fused, device=dev, dtype=bf)
+    inv = torch.rand(RD // 2, device=dev)
+    kz, vz = torch.zeros(nb, 1, BS, KD, device=dev, dtype=bf), torch.zeros(nb, 1, R, BS, device=dev, dtype=bf)
+    wn = torch.ones(R, device=dev)
+    t = _graph_time(lambda: ops.latent_kv_write(y, 768, R, RD, wn, 1e-5, meta.positions, meta.slots, inv, 1.2, kz, vz), iters=50)
+    out["cache_write"] = {"mabivik_ms": round(t * 1e3, 4), "mabivik_roof_frac": _roof(0, T * (KD + KD + R) * 2, t)}
+    width = (H + G) * 128 + G * 128
+    y2 = torch.randn(T, width, device=dev, dtype=bf)
+    qn, kn = torch.ones(H * 128, device=dev), torch.ones(G * 128, device=dev)
+    inv2, vinv = torch.rand(32, device=dev), torch.rand(64, device=dev)
+    kp, vp = torch.zeros(nb, G, BS, 128, device=dev, dtype=bf), torch.zeros(nb, G, 128, BS, device=dev, dtype=bf)
+    t = _graph_time(lambda: ops.rope_pairs_kv_write(y2, meta.positions, meta.slots, H, G, 128, 128, qn, kn, 1e-5, inv2, vinv, kp, vp), iters=50)
+    out["cache_write"].update({"padadra_ms": round(t * 1e3, 4), "padadra_roof_frac": _roof(0, T * width * 2 * 2, t)})
+    # ---- query assembly: tail rotary into the packed query (the per-head products are vendor GEMMs) ----
+    qsrc, qdst = torch.randn(T, H, 128 + RD, device=dev, dtype=bf), torch.empty(T, H, KD, device=dev, dtype=bf)
+    t = _graph_time(lambda: ops.rope_half_tail(qsrc, 128, qdst, R, meta.positions, inv, 1.2), iters=50)
+    out["query_tail_rotary"] = {"mabivik_ms": round(t * 1e3, 4), "mabivik_roof_frac": _roof(0, T * H * RD * 2 * 2, t)}
+    # ---- routed experts: gated (three matrices, activation in the epilogue) against relu^2 (two matrices) ----
+    E, top, ff = 8, 2, s["ff"] // 4
+    for name, rows_ in (("prefill", 8192), ("decode", 64)):
+        h = torch.randn(rows_, W, device=dev, dtype=bf)
+        up2 = torch.randn(E, 2 * ff, W, device=dev, dtype=bf) * 0.02
+        up1 = torch.randn(E, ff, W, device=dev, dtype=bf) * 0.02
+        down = torch.randn(E, W, ff, device=dev, dtype=bf) * 0.02
+        idx = torch.randint(0, E, (rows_, 1), device=dev, dtype=torch.int32)
+        idx = torch.cat([idx, (idx + 1 + torch.randint(0, E - 1, (rows_, 1), device=dev, dtype=torch.int32)) % E], 1).contiguous()
+        wts = torch.full((rows_, top), 0.5, device=dev)
+        act = rows_ * W * 2 * (2 + 2 * top)
+        t = _time(lambda: ops.moe_experts(h, up2, down, idx, wts, "silu_gated"), iters=20)
+        out[f"experts_{name}"] = {"mabivik_ms": round(t * 1e3, 4),
+                                  "mabivik_roof_frac": _roof(2 * 3 * rows_ * top * ff * W, 3 * E * ff * W * 2 + act, t)}
+        t = _time(lambda: ops.moe_experts(h, up1, down, idx, wts, "relu2"), iters=20)
+        out[f"experts_{name}"].update({"mofidra_ms": round(t * 1e3, 4),
+                                       "mofidra_roof_frac": _roof(2 * 2 * rows_ * top * ff * W, 2 * E * ff * W * 2 + act, t)})
+    # ---- the recurrences: one decay per head (delta rule; state space with scaled writes) against one per channel ----
+    Gq = max(1, H // 2)
+    Hs = 2 * W // 128
+    for name, rows_, m_ in (("prefill", T, meta), ("decode", b, dmeta)):
+        nseq = m_.q_start.numel() - 1
+        m_.state_rows = torch.arange(nseq, dtype=torch.int32, device=dev)
+        q32, k32 = torch.randn(rows_, Gq, 128, device=dev) * 0.1, torch.randn(rows_, Gq, 128, device=dev) * 0.1
+        g1, gc, beta = torch.rand(rows_, H, 1, device=dev), torch.rand(rows_, H, 128, device=dev), torch.rand(rows_, H, device=dev)
+        v = torch.randn(rows_, H * 128, device=dev, dtype=bf)
+        S = torch.zeros(max(n, b) + 1, H, 128, 128, device=dev)
+        timer = (lambda f: _time(f, iters=10)) if name == "prefill" else (lambda f: _graph_time(f, iters=50))
+        flops = rows_ * H * 128 * 128 * 8
+        io = rows_ * (2 * Gq * 128 * 4 + H * 4 + H * 128 * 2 + H * 128 * 4) + nseq * H * 128 * 128 * 4 * 2
+        t = timer(lambda: ops.gated_state_scan(q32, k32, g1, v, beta, m_, S, True))
+        entry = {"mabivik_ms": round(t * 1e3, 4), "mabivik_roof_frac": round(max(flops / PEAK_VALU, io / PEAK_BW) / t, 4)}
+        t = timer(lambda: ops.gated_state_scan(q32, k32, gc, v, beta, m_, S, True))
+        entry.update({"padadra_ms": round(t * 1e3, 4),
+                      "padadra_roof_frac": round(max(flops / PEAK_VALU, (io + rows_ * H * 127 * 4) / PEAK_BW) / t, 4)})
+        out[f"delta_scan_{name}"] = entry
+        qs, ks = torch.randn(rows_, 2, 128, device=dev) * 0.1, torch.randn(rows_, 2, 128, device=dev) * 0.1
+        gs, dts = torch.rand(rows_, Hs, 1, device=dev), torch.rand(rows_, Hs, device=dev)
+        vs = torch.randn(rows_, Hs * 128, device=dev, dtype=bf)
+        Ss = torch.zeros(max(n, b) + 1, Hs, 128, 128, device=dev)
+        t = timer(lambda: ops.gated_state_scan(qs, ks, gs, vs, dts, m_, Ss, False))
+        flops = rows_ * Hs * 128 * 128 * 6
+        io = rows_ * (2 * 2 * 128 * 4 + Hs * 8 + Hs * 128 * 2 + Hs * 128 * 4) + nseq * Hs * 128 * 128 * 4 * 2
+        out[f"ssm_scan_{name}"] = {"mabivik_ms": round(t * 1e3, 4), "mabivik_roof_frac": round(max(flops / PEAK_VALU, io / PEAK_BW) / t, 4)}
+    # ---- output norms of the recurrent mixers, 8192 rows ----
+    o32 = torch.randn(T, Hs, 128, device=dev)
+    skip, z = torch.randn(T, Hs * 128, device=dev, dtype=bf), torch.randn(T, Hs * 128, device=dev, dtype=bf)
+    D, wg = torch.randn(Hs, device=dev), torch.randn(Hs * 128, device=dev)
+    t = _time(lambda: ops.gated_group_norm(o32, skip, D, z, wg, 2, 1e-5, bf), iters=20)
+    out["recurrent_out_norm"] = {"mabivik_ms": round(t * 1e3, 4), "mabivik_roof_frac": _roof(0, T * Hs * 128 * (4 + 2 + 2 + 2), t)}
+    wh = torch.randn(128, device=dev)
+    t = _time(lambda: ops.head_norm_gate(o32, wh, 1e-5, z, bf), iters=20)
+    out["recurrent_out_norm"].update({"padadra_ms": round(t * 1e3, 4), "padadra_roof_frac": _roof(0, T * Hs * 128 * (4 + 2 + 2), t)})
+    # ---- short convolution with bias, 8192 rows ----
+    cc = Hs * 128 + 2 * 2 * 128
+    yc, cw, cb = torch.randn(T, cc, device=dev, dtype=bf), torch.randn(cc, 4, device=dev), torch.randn(cc, device=dev)
+    cstate = torch.zeros(n + 1, 3, cc, device=dev, dtype=bf)
+    t = _time(lambda: ops.short_conv(yc, cc, cw, meta, cstate, "silu", cb), iters=20)
+    out["short_conv"] = {"mabivik_ms": round(t * 1e3, 4), "mabivik_roof_frac": _roof(0, T * cc * 2 * 2, t)}
+    t = _time(lambda: ops.short_conv(yc, cc, cw, meta, cstate, "silu"), iters=20)
+    out["short_conv"].update({"padadra_ms": round(t * 1e3, 4), "padadra_roof_frac": _roof(0, T * cc * 2 * 2, t)})
+    return out
+
+
 def run(sizes=("w2048", "w4096"), kernels=True) -> dict:
     dev = torch.device("cuda", torch.cuda.current_device())
     ops = get_ops("hip")
@@ -312,6 +486,7 @@ def run(sizes=("w2048", "w4096"), kernels=True) -> dict:
             for label, build in (("mofidra_dense", lambda: MofidraModel(mofidra_config(s, False), ops, dev)),
                                  ("mofidra_moe", lambda: MofidraModel(mofidra_config(s, True), ops, dev)),
                                  ("padadra", lambda: PadadraModel(padadra_config(s), ops, dev)),
+                                 ("mabivik", lambda: MabivikModel(mabivik_config(s), ops, dev)),
                                  ("decoder", lambda: DecoderModel(decoder_config(s), ops, dev))):
                 model = build()
                 model.init_random(seed=1, std=0.02)
@@ -321,6 +496,7 @@ def run(sizes=("w2048", "w4096"), kernels=True) -> dict:
             if kernels:
                 entry["kernels"] = kernel_pairs(s, dev)
                 entry["state_kernels"] = state_kernels(s, dev)
+                entry["latent_kernels"] = latent_kernels(s, dev)
             result["sizes"][name] = entry
     return result
 

@@ -324,7 +324,7 @@ __global__ __launch_bounds__(64, OCC) void decode_mfma_kernel(AttnArgs a) {
   const int row = a.work ? a.work[2 * item] : item, seq = a.work ? a.work[2 * item + 1] : item;
   const int ctx = a.seq_lens[seq];
   const int lo = a.window > 0 ? max(0, ctx - a.window) : 0;          // first visible key
-  const int split_abs = lo / SPLIT_KEYS + split;                      // splits count from the window's first
+  const int split_abs = lo / SPLIT_KEYS + split;                    // splits count from the window's first
   const int k_end = min(ctx, (split_abs + 1) * SPLIT_KEYS);
   const int k_begin = max(split_abs * SPLIT_KEYS, lo & ~15);
   if (k_begin >= k_end) return;

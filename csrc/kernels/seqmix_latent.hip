@@ -60,7 +60,7 @@ __global__ __launch_bounds__(NT) void embed_scale_dyt_kernel(const int* __restri
 // ---------------------------------------------------------------- x += post(y); out = pre(x)
 // POST 0: dynamic tanh of y; 1: y / sqrt(mean(y^2) + eps) * w.  PRE 0: nothing; 1: x rounded to T;
 // 2: dynamic tanh of the new x.  Y is the type of the sublayer output (T, or float for the fp32
-// sum of the experts).  ROWS_VEC: 4 consecutive columns per thread (W a multiple of 4).
+// sum of the experts).
 template <typename T, typename Y, int POST>
 __global__ __launch_bounds__(NT) void residual_post_norm_kernel(float* __restrict__ resid, const Y* __restrict__ y, Dyt post,
                                                                 float eps, int pre_kind, Dyt pre, T* __restrict__ out, int W) {
@@ -101,7 +101,8 @@ __global__ __launch_bounds__(NT) void rmsnorm_cols_kernel(const T* __restrict__ 
 }
 
 // ---------------------------------------------------------------- latent + shared rotated key part -> pages
-// One block per token.  Columns off .. off + R - 1 of the row are the latent (RMS norm, weight w),
+// One wave per token (a row is a few hundred features: no block-wide reduction, four tokens per
+// workgroup).  Columns off .. off + R - 1 of the row are the latent (RMS norm, weight w),
 // the next RD the shared key part (the first 2 half of them turned by position * inv_freq, times
 // amp).  K slab of the token's page: features [latent | key part]; V^T slab: the latent.
 template <typename T>
@@ -110,16 +111,17 @@ __global__ __launch_bounds__(NT) void latent_kv_write_kernel(const T* __restrict
                                                              const int* __restrict__ positions, const int* __restrict__ slots,
                                                              const float* __restrict__ inv_freq, int half, float amp,
                                                              T* __restrict__ k_cache, T* __restrict__ v_cache, int BS,
-                                                             int num_blocks) {
-  __shared__ float red[NT / 64];
-  const int t = blockIdx.x;
+                                                             int num_blocks, int T_) {
+  const int lane = threadIdx.x & 63;
+  const int t = blockIdx.x * (NT / 64) + (threadIdx.x >> 6);
+  if (t >= T_) return;
   const T* row = y + static_cast<size_t>(t) * stride + off;
   float ss = 0.f;
-  for (int i = threadIdx.x; i < R; i += NT) {
+  for (int i = lane; i < R; i += 64) {
     const float v = Elem<T>::ld(row[i]);
     ss += v * v;
   }
-  const float r = 1.0f / sqrtf(block_sum(ss, red) / R + eps);
+  const float r = 1.0f / sqrtf(wave_sum(ss) / R + eps);
   const int slot = slots[t];
   const int blk = slot / BS, o = slot - blk * BS;
   if (slot < 0 || blk >= num_blocks) return;
@@ -128,7 +130,7 @@ __global__ __launch_bounds__(NT) void latent_kv_write_kernel(const T* __restrict
   T* ks = k_cache + static_cast<size_t>(blk) * BS * KD;
   T* vs = v_cache + static_cast<size_t>(blk) * R * BS;
   const float pos = static_cast<float>(positions[t]);
-  for (int i = threadIdx.x; i < KD; i += NT) {
+  for (int i = lane; i < KD; i += 64) {
     float val;
     if (i < R) {
       val = Elem<T>::ld(row[i]) * r * w[i];
@@ -154,27 +156,32 @@ __global__ __launch_bounds__(NT) void latent_kv_write_kernel(const T* __restrict
 }
 
 // dst[t, h, dst_off + j] = turn(src[t, h, src_off + j]), j < n: the first 2 half features of the
-// tail turn by position * inv_freq (j pairs with j + half), the others are copied.
+// tail turn by position * inv_freq (j pairs with j + half), the others are copied.  A thread owns
+// one pair (or one copied feature) of a token and walks the heads: one sincos serves all of them.
 template <typename T>
 __global__ __launch_bounds__(NT) void rope_half_tail_kernel(const T* __restrict__ src, int Ds, int src_off, T* __restrict__ dst,
                                                             int Dd, int dst_off, int n, const int* __restrict__ positions,
                                                             const float* __restrict__ inv_freq, int half, float amp,
                                                             int64_t total, int H) {
+  const int per = n - half;   // work items of a token: `half` pairs, then the copied features
   for (int64_t e = static_cast<int64_t>(blockIdx.x) * NT + threadIdx.x; e < total; e += static_cast<int64_t>(gridDim.x) * NT) {
-    const int j = static_cast<int>(e % n);
-    const int64_t th = e / n;
-    const T* s = src + th * Ds + src_off;
-    float val = Elem<T>::ld(s[j]);
-    if (j < 2 * half) {
-      const int f = j < half ? j : j - half;
+    const int64_t t = e / per;
+    const int j = static_cast<int>(e - t * per);
+    const T* s = src + t * H * Ds + src_off;
+    T* d = dst + t * H * Dd + dst_off;
+    if (j < half) {
       float sn, cs;
-      sincosf(static_cast<float>(positions[th / H]) * inv_freq[f], &sn, &cs);
+      sincosf(static_cast<float>(positions[t]) * inv_freq[j], &sn, &cs);
       sn *= amp;
       cs *= amp;
-      const float other = Elem<T>::ld(s[j < half ? j + half : j - half]);
-      val = j < half ? val * cs - other * sn : val * cs + other * sn;
+      for (int h = 0; h < H; ++h) {
+        const float a = Elem<T>::ld(s[h * Ds + j]), b = Elem<T>::ld(s[h * Ds + j + half]);
+        d[h * Dd + j] = Elem<T>::st(a * cs - b * sn);
+        d[h * Dd + j + half] = Elem<T>::st(b * cs + a * sn);
+      }
+    } else {
+      for (int h = 0; h < H; ++h) d[h * Dd + j + half] = s[h * Ds + j + half];
     }
-    dst[th * Dd + dst_off + j] = Elem<T>::st(val);
   }
 }
 
@@ -330,10 +337,11 @@ BCG_API int bcg_latent_kv_write(const void* y, int64_t stride, int off, int R, i
   hipStream_t s = static_cast<hipStream_t>(stream);
   const float *wf = static_cast<const float*>(w), *fr = static_cast<const float*>(inv_freq);
   const int *ps = static_cast<const int*>(positions), *sl = static_cast<const int*>(slots);
-  BCG_BY_TYPE((latent_kv_write_kernel<float><<<T_, NT, 0, s>>>(static_cast<const float*>(y), stride, off, R, RD, wf, eps, ps, sl, fr, half, amp,
-                                                              static_cast<float*>(k_cache), static_cast<float*>(v_cache), BS, num_blocks)),
-              (latent_kv_write_kernel<bf16_t><<<T_, NT, 0, s>>>(static_cast<const bf16_t*>(y), stride, off, R, RD, wf, eps, ps, sl, fr, half, amp,
-                                                               static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), BS, num_blocks)));
+  const int grid = (T_ + NT / 64 - 1) / (NT / 64);
+  BCG_BY_TYPE((latent_kv_write_kernel<float><<<grid, NT, 0, s>>>(static_cast<const float*>(y), stride, off, R, RD, wf, eps, ps, sl, fr, half, amp,
+                                                                static_cast<float*>(k_cache), static_cast<float*>(v_cache), BS, num_blocks, T_)),
+              (latent_kv_write_kernel<bf16_t><<<grid, NT, 0, s>>>(static_cast<const bf16_t*>(y), stride, off, R, RD, wf, eps, ps, sl, fr, half, amp,
+                                                                 static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), BS, num_blocks, T_)));
   return BCG_CHECK_LAUNCH();
 }
 
@@ -343,7 +351,7 @@ BCG_API int bcg_rope_half_tail(const void* src, int Ds, int src_off, void* dst, 
   if (T_ <= 0 || H <= 0 || n <= 0) return 0;
   if (n != Dd - dst_off || 2 * half > n) return -2;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int64_t total = static_cast<int64_t>(T_) * H * n;
+  const int64_t total = static_cast<int64_t>(T_) * (n - half);
   const int* ps = static_cast<const int*>(positions);
   const float* fr = static_cast<const float*>(inv_freq);
   BCG_BY_TYPE((rope_half_tail_kernel<float><<<ew_grid(total), NT, 0, s>>>(static_cast<const float*>(src), Ds, src_off, static_cast<float*>(dst), Dd,

@@ -103,6 +103,7 @@ def case(request, tmp_path_factory):
     cfg = C.CASES[name]
     sd = O.to_f64(C.checkpoint(cfg, path, seed=len(name)))
     e = K.Env("hip", "cuda", getattr(torch, dtype))
+    e.measure_noise(path, cfg, sd)
     eng = C.engine(path, backend="hip", dtype=e.dtype, pool_tokens=320)
     assert eng.ops.name == "hip"
     yield e, cfg, sd, eng
