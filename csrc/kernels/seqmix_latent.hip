@@ -61,6 +61,53 @@ __global__ __launch_bounds__(NT) void embed_scale_dyt_kernel(const int* __restri
 // POST 0: dynamic tanh of y; 1: y / sqrt(mean(y^2) + eps) * w.  PRE 0: nothing; 1: x rounded to T;
 // 2: dynamic tanh of the new x.  Y is the type of the sublayer output (T, or float for the fp32
 // sum of the experts).
+template <typename T> struct Vec4 { typedef f32x4 type; };
+template <> struct Vec4<bf16_t> { typedef u16x4 type; };
+
+// The same with four consecutive columns per thread (W a multiple of 4, every pointer 16-byte
+// aligned): 8- / 16-byte loads and stores.
+template <typename T, typename Y, int POST>
+__global__ __launch_bounds__(NT) void residual_post_norm_vec_kernel(float* __restrict__ resid, const Y* __restrict__ y, Dyt post,
+                                                                    float eps, int pre_kind, Dyt pre, T* __restrict__ out, int W) {
+  typedef typename Vec4<T>::type VT;
+  typedef typename Vec4<Y>::type VY;
+  __shared__ float red[NT / 64];
+  const size_t base = static_cast<size_t>(blockIdx.x) * W;
+  float r = 1.0f;
+  if (POST == 1) {
+    float ss = 0.f;
+    for (int i = 4 * threadIdx.x; i < W; i += 4 * NT) {
+      const VY v = *reinterpret_cast<const VY*>(y + base + i);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float f = Elem<Y>::ld(v[j]);
+        ss += f * f;
+      }
+    }
+    r = 1.0f / sqrtf(block_sum(ss, red) / W + eps);
+  }
+  for (int i = 4 * threadIdx.x; i < W; i += 4 * NT) {
+    const VY v = *reinterpret_cast<const VY*>(y + base + i);
+    f32x4 x = *reinterpret_cast<const f32x4*>(resid + base + i);
+    const f32x4 pw = *reinterpret_cast<const f32x4*>(post.w + i);
+    f32x4 pb = {0.f, 0.f, 0.f, 0.f}, qw = pb, qb = pb;
+    if (POST == 0) pb = *reinterpret_cast<const f32x4*>(post.b + i);
+    if (pre_kind == 2) {
+      qw = *reinterpret_cast<const f32x4*>(pre.w + i);
+      qb = *reinterpret_cast<const f32x4*>(pre.b + i);
+    }
+    VT o;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float f = Elem<Y>::ld(v[j]);
+      x[j] += POST == 0 ? tanhf(post.alpha * f) * pw[j] + pb[j] : f * r * pw[j];
+      o[j] = Elem<T>::st(pre_kind == 2 ? tanhf(pre.alpha * x[j]) * qw[j] + qb[j] : x[j]);
+    }
+    *reinterpret_cast<f32x4*>(resid + base + i) = x;
+    if (pre_kind != 0) *reinterpret_cast<VT*>(out + base + i) = o;
+  }
+}
+
 template <typename T, typename Y, int POST>
 __global__ __launch_bounds__(NT) void residual_post_norm_kernel(float* __restrict__ resid, const Y* __restrict__ y, Dyt post,
                                                                 float eps, int pre_kind, Dyt pre, T* __restrict__ out, int W) {
@@ -157,30 +204,34 @@ __global__ __launch_bounds__(NT) void latent_kv_write_kernel(const T* __restrict
 
 // dst[t, h, dst_off + j] = turn(src[t, h, src_off + j]), j < n: the first 2 half features of the
 // tail turn by position * inv_freq (j pairs with j + half), the others are copied.  A thread owns
-// one pair (or one copied feature) of a token and walks the heads: one sincos serves all of them.
+// one pair (or one copied feature) of a token for `hpt` heads: with hpt = H one sincos serves all
+// heads of a token (large steps), with hpt = 1 every head has a thread of its own (small steps).
 template <typename T>
 __global__ __launch_bounds__(NT) void rope_half_tail_kernel(const T* __restrict__ src, int Ds, int src_off, T* __restrict__ dst,
                                                             int Dd, int dst_off, int n, const int* __restrict__ positions,
                                                             const float* __restrict__ inv_freq, int half, float amp,
-                                                            int64_t total, int H) {
-  const int per = n - half;   // work items of a token: `half` pairs, then the copied features
+                                                            int64_t total, int H, int hpt) {
+  const int per = n - half;   // work items of a (token, head chunk): `half` pairs, then the copied features
+  const int chunks = H / hpt;
   for (int64_t e = static_cast<int64_t>(blockIdx.x) * NT + threadIdx.x; e < total; e += static_cast<int64_t>(gridDim.x) * NT) {
-    const int64_t t = e / per;
-    const int j = static_cast<int>(e - t * per);
-    const T* s = src + t * H * Ds + src_off;
-    T* d = dst + t * H * Dd + dst_off;
+    const int64_t tc = e / per;
+    const int j = static_cast<int>(e - tc * per);
+    const int64_t t = tc / chunks;
+    const int h0 = static_cast<int>(tc - t * chunks) * hpt;
+    const T* s = src + (t * H + h0) * Ds + src_off;
+    T* d = dst + (t * H + h0) * Dd + dst_off;
     if (j < half) {
       float sn, cs;
       sincosf(static_cast<float>(positions[t]) * inv_freq[j], &sn, &cs);
       sn *= amp;
       cs *= amp;
-      for (int h = 0; h < H; ++h) {
+      for (int h = 0; h < hpt; ++h) {
         const float a = Elem<T>::ld(s[h * Ds + j]), b = Elem<T>::ld(s[h * Ds + j + half]);
         d[h * Dd + j] = Elem<T>::st(a * cs - b * sn);
         d[h * Dd + j + half] = Elem<T>::st(b * cs + a * sn);
       }
     } else {
-      for (int h = 0; h < H; ++h) d[h * Dd + j + half] = s[h * Ds + j + half];
+      for (int h = 0; h < hpt; ++h) d[h * Dd + j + half] = s[h * Ds + j + half];
     }
   }
 }
@@ -303,9 +354,17 @@ BCG_API int bcg_residual_post_norm(void* resid, const void* y, int y_f32, int po
   const Dyt post{post_alpha, static_cast<const float*>(post_w), static_cast<const float*>(post_b)};
   const Dyt pre{pre_alpha, static_cast<const float*>(pre_w), static_cast<const float*>(pre_b)};
   float* x = static_cast<float*>(resid);
+  auto al16 = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+  const bool vec = W % 4 == 0 && al16(resid) && al16(y) && al16(out) && al16(post_w) && al16(post_b) && al16(pre_w) && al16(pre_b);
 #define BCG_RPN(TYPE, YTYPE)                                                                                                  \
   do {                                                                                                                        \
-    if (post_kind == 0)                                                                                                       \
+    if (vec && post_kind == 0)                                                                                                \
+      residual_post_norm_vec_kernel<TYPE, YTYPE, 0><<<T_, NT, 0, s>>>(x, static_cast<const YTYPE*>(y), post, eps, pre_kind,  \
+                                                                      pre, static_cast<TYPE*>(out), W);                       \
+    else if (vec)                                                                                                             \
+      residual_post_norm_vec_kernel<TYPE, YTYPE, 1><<<T_, NT, 0, s>>>(x, static_cast<const YTYPE*>(y), post, eps, pre_kind,  \
+                                                                      pre, static_cast<TYPE*>(out), W);                       \
+    else if (post_kind == 0)                                                                                                  \
       residual_post_norm_kernel<TYPE, YTYPE, 0><<<T_, NT, 0, s>>>(x, static_cast<const YTYPE*>(y), post, eps, pre_kind, pre, \
                                                                   static_cast<TYPE*>(out), W);                                \
     else                                                                                                                      \
@@ -351,13 +410,14 @@ BCG_API int bcg_rope_half_tail(const void* src, int Ds, int src_off, void* dst, 
   if (T_ <= 0 || H <= 0 || n <= 0) return 0;
   if (n != Dd - dst_off || 2 * half > n) return -2;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int64_t total = static_cast<int64_t>(T_) * (n - half);
+  const int hpt = static_cast<int64_t>(T_) * (n - half) >= (1 << 16) ? H : 1;
+  const int64_t total = static_cast<int64_t>(T_) * (H / hpt) * (n - half);
   const int* ps = static_cast<const int*>(positions);
   const float* fr = static_cast<const float*>(inv_freq);
   BCG_BY_TYPE((rope_half_tail_kernel<float><<<ew_grid(total), NT, 0, s>>>(static_cast<const float*>(src), Ds, src_off, static_cast<float*>(dst), Dd,
-                                                                         dst_off, n, ps, fr, half, amp, total, H)),
+                                                                         dst_off, n, ps, fr, half, amp, total, H, hpt)),
               (rope_half_tail_kernel<bf16_t><<<ew_grid(total), NT, 0, s>>>(static_cast<const bf16_t*>(src), Ds, src_off, static_cast<bf16_t*>(dst), Dd,
-                                                                          dst_off, n, ps, fr, half, amp, total, H)));
+                                                                          dst_off, n, ps, fr, half, amp, total, H, hpt)));
   return BCG_CHECK_LAUNCH();
 }
 

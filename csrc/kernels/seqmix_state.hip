@@ -168,8 +168,9 @@ __global__ __launch_bounds__(NT) void short_conv_kernel(const T* __restrict__ y,
   out[static_cast<size_t>(t) * C + c] = Elem<T>::st(acc);
 }
 
-// The same for VEC consecutive channels per thread (one 16-byte load per tap) and CONV_ROWS
-// consecutive rows per block, the thread's TAPS x VEC weights in registers.  Needs C, the row
+// The same for VEC consecutive channels per thread (one 16-byte load per tap) and `rows`
+// consecutive rows per block (CONV_ROWS in large steps, where a thread's weights are worth keeping;
+// one in small steps, which need the blocks), the thread's TAPS x VEC weights in registers.  Needs C, the row
 // strides and the base addresses to be multiples of VEC elements.
 constexpr int CONV_ROWS = 8;
 
@@ -179,7 +180,7 @@ __global__ __launch_bounds__(NT) void short_conv_vec_kernel(const T* __restrict_
                                                             const int* __restrict__ token_seq, const int* __restrict__ q_start,
                                                             const int* __restrict__ state_rows, const T* __restrict__ state,
                                                             int n_rows, T* __restrict__ out, int act, int T_,
-                                                            const float* __restrict__ bias) {
+                                                            const float* __restrict__ bias, int rows) {
   struct alignas(sizeof(T) * VEC) Vec { T e[VEC]; };
   const int c = (blockIdx.y * NT + threadIdx.x) * VEC;
   if (c >= C) return;
@@ -190,8 +191,8 @@ __global__ __launch_bounds__(NT) void short_conv_vec_kernel(const T* __restrict_
 #pragma unroll
     for (int j = 0; j < TAPS; ++j) wr[e][j] = w[static_cast<size_t>(c + e) * TAPS + j];
   }
-  const int t_end = min(T_, (static_cast<int>(blockIdx.x) + 1) * CONV_ROWS);
-  for (int t = blockIdx.x * CONV_ROWS; t < t_end; ++t) {
+  const int t_end = min(T_, (static_cast<int>(blockIdx.x) + 1) * rows);
+  for (int t = blockIdx.x * rows; t < t_end; ++t) {
     const int seg = token_seq[t], off = t - q_start[seg], pos = positions[t];
     const int sr = state_rows[seg];
     const bool row_ok = sr >= 0 && sr < n_rows;
@@ -226,10 +227,11 @@ bool launch_conv_vec(const T* y, int64_t y_stride, int C, const float* w, int ta
   constexpr int VEC = 16 / sizeof(T);
   const uintptr_t bits = reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(state) | reinterpret_cast<uintptr_t>(out);
   if (C % VEC || y_stride % VEC || bits % 16 || taps < 2 || taps > 4) return false;
-  dim3 grid((T_ + CONV_ROWS - 1) / CONV_ROWS, (C / VEC + NT - 1) / NT);
-  if (taps == 2) short_conv_vec_kernel<T, VEC, 2><<<grid, NT, 0, s>>>(y, y_stride, C, w, ps, ts, qs, sr, state, n_rows, out, act, T_, bias);
-  else if (taps == 3) short_conv_vec_kernel<T, VEC, 3><<<grid, NT, 0, s>>>(y, y_stride, C, w, ps, ts, qs, sr, state, n_rows, out, act, T_, bias);
-  else short_conv_vec_kernel<T, VEC, 4><<<grid, NT, 0, s>>>(y, y_stride, C, w, ps, ts, qs, sr, state, n_rows, out, act, T_, bias);
+  const int rows = T_ >= 2048 ? CONV_ROWS : 1;
+  dim3 grid((T_ + rows - 1) / rows, (C / VEC + NT - 1) / NT);
+  if (taps == 2) short_conv_vec_kernel<T, VEC, 2><<<grid, NT, 0, s>>>(y, y_stride, C, w, ps, ts, qs, sr, state, n_rows, out, act, T_, bias, rows);
+  else if (taps == 3) short_conv_vec_kernel<T, VEC, 3><<<grid, NT, 0, s>>>(y, y_stride, C, w, ps, ts, qs, sr, state, n_rows, out, act, T_, bias, rows);
+  else short_conv_vec_kernel<T, VEC, 4><<<grid, NT, 0, s>>>(y, y_stride, C, w, ps, ts, qs, sr, state, n_rows, out, act, T_, bias, rows);
   return true;
 }
 
