@@ -146,8 +146,8 @@ def seqmix_ops(lib, linear):
         dim = qd // maps
         G = k_cache.shape[1]
         NB, BS = _cache_ok(k_cache, v_cache, G, qd, vdim, q.dtype)
-        _req(H % G == 0 and maps in (1, 2) and dim <= (256 if maps == 1 else 128) and vdim <= 256,
-             "multimap attention: maps <= 2, dim <= 128 (one map: 256), vdim <= 256")
+        _req(H % G == 0 and maps in (1, 2) and dim <= (512 if maps == 1 else 128) and vdim <= 256,
+             "multimap attention: maps <= 2, dim <= 128 (one map: 512), vdim <= 256")
         bt = meta.block_tables
         lens = meta.seq_lens if meta.attn_seq_lens is None else meta.attn_seq_lens
         _req(bt.dtype == torch.int32 and bt.dim() == 2 and bt.is_contiguous() and lens.dtype == torch.int32

@@ -455,8 +455,10 @@ int launch_prefill(const AttnArgs& a, int n_tiles, int tile_rows, hipStream_t s)
     else prefill_kernel<T, 4, 8, 1, false, false, 2><<<grid, 256, 0, s>>>(a);
   } else if (a.dim <= 128) {   // (the branch-free form of the wide instance runs out of registers)
     prefill_kernel<T, 8, 16, 1, false, false, 1><<<grid, 256, 0, s>>>(a);
-  } else {   // one map of up to 256 key features (a latent plus a rotated part)
+  } else if (a.dim <= 256) {   // one map of up to 256 key features (a latent plus a rotated part)
     prefill_kernel<T, 16, 16, 1, false, false, 1, 0, 1><<<grid, 256, 0, s>>>(a);
+  } else {   // ... up to 512 (slow: the fragments of a row fill the register file)
+    prefill_kernel<T, 32, 16, 1, false, false, 1, 0, 1><<<grid, 256, 0, s>>>(a);
   }
   return BCG_CHECK_LAUNCH();
 }
@@ -498,8 +500,10 @@ int launch_decode(const AttnArgs& a, int n_items, hipStream_t s) {
     else decode_mfma_kernel<T, 4, 8, 1, false, false, 2><<<grid, 64, 0, s>>>(a);
   } else if (a.dim <= 128) {
     decode_mfma_kernel<T, 8, 16, 1, false, false, 1><<<grid, 64, 0, s>>>(a);
-  } else {
+  } else if (a.dim <= 256) {
     decode_mfma_kernel<T, 16, 16, 1, false, false, 1, 0, 1><<<grid, 64, 0, s>>>(a);
+  } else {
+    decode_mfma_kernel<T, 32, 16, 1, false, false, 1, 0, 1><<<grid, 64, 0, s>>>(a);
   }
   if (a.vdim <= 128) decode_merge_kernel<T, 2><<<dim3(a.H, n_items), 64, 0, s>>>(a);
   else decode_merge_kernel<T, 4><<<dim3(a.H, n_items), 64, 0, s>>>(a);
@@ -519,7 +523,7 @@ BCG_API int bcg_multimap_attention(int mode, const void* q, const void* k_cache,
                                    float out_scale, int tile_rows, int is_f32, int window, const void* sink, void* stream) {
   if (n_work <= 0) return 0;
   if ((window > 0 || sink != nullptr) && maps != 1) return -2;
-  if (maps < 1 || maps > 2 || dim > (maps == 1 ? 256 : 128) || vdim > 256 || BS % 16 || H % G || n_work > 65535 * 16) return -2;
+  if (maps < 1 || maps > 2 || dim > (maps == 1 ? 512 : 128) || vdim > 256 || BS % 16 || H % G || n_work > 65535 * 16) return -2;
   AttnArgs a;
   a.q = q; a.k_cache = k_cache; a.v_cache = v_cache;
   a.block_tables = static_cast<const int*>(block_tables); a.q_start = static_cast<const int*>(q_start);

@@ -40,10 +40,10 @@ def test_latent_attention_whole_and_in_portions(env, name):
 
 
 def test_latent_attention_exact_and_wide_shapes(env):
-    """Cached rows on the 16-wide MFMA grid (the straight-line instances), one of 160 and one of
-    256 features (the wide one-map instance), several 64-row tiles and decode splits."""
+    """Cached rows on the 16-wide MFMA grid (the straight-line instances), of 160 and 256 features
+    (the wide one-map instance) and of 320 (the widest), several 64-row tiles and decode splits."""
     for heads, dim, rot, vdim, rank, window in [(4, 32, 32, 32, 64, 70), (2, 64, 32, 48, 128, 150), (3, 48, 64, 32, 192, 0),
-                                                (17, 16, 16, 16, 32, 40)]:
+                                                (17, 16, 16, 16, 32, 40), (2, 32, 64, 24, 256, 90)]:
         layers = [C.layer("latent_attention", C.latent(heads, dim, rot, vdim, 24, rank, window), 0)]
         got, want = K.run_mixer(env, layers, 200, [150, 1, 1, 40, 1, 1, 1, 1, 1, 1, 1, 1], seed=heads, width=48)
         env.close(got, want)
