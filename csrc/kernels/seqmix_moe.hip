@@ -304,6 +304,99 @@ __global__ __launch_bounds__(256) void moe_gemm_lds_kernel(const T* __restrict__
   }
 }
 
+// The LDS-staged product for small steps: a workgroup covers 64 columns instead of 256 (wave w takes
+// the 16 rows of m-tile w times all 64 columns), so a decode step's few position tiles become four
+// times as many workgroups; the staging and the fragment layout are those of `moe_gemm_lds_kernel`.
+template <typename T>
+__global__ __launch_bounds__(256) void moe_gemm_lds_narrow_kernel(const T* __restrict__ a, int64_t a_stride,
+                                                                  const T* __restrict__ w, T* __restrict__ out,
+                                                                  int64_t out_stride, const int* __restrict__ sorted,
+                                                                  const int* __restrict__ tile_expert, int N, int K, int top,
+                                                                  int gather, int scatter, int act) {
+  typedef typename Elem<T>::frag F;
+  constexpr int BK = 32, LDK = BK + 8, TNN = 64;
+  typedef T Chunk __attribute__((ext_vector_type(8)));
+  __shared__ __attribute__((aligned(16))) T As[TM * LDK];
+  __shared__ __attribute__((aligned(16))) T Ws[TNN * LDK];
+  const int e = tile_expert[blockIdx.x];
+  if (e < 0) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 15, grp = lane >> 4;
+  const int p0 = blockIdx.x * TM, nb = blockIdx.y * TNN;
+  const T* we = w + static_cast<size_t>(e) * N * K;
+  const int s_row = tid >> 2, s_k = (tid & 3) * 8;
+  const int a_slot = sorted[p0 + s_row];
+  const T* a_src = a + (gather ? static_cast<int64_t>(a_slot < 0 ? 0 : a_slot / top) : static_cast<int64_t>(p0 + s_row)) * a_stride + s_k;
+  const bool w_ok = nb + s_row < N;
+  const T* w_src = we + static_cast<size_t>(w_ok ? nb + s_row : 0) * K + s_k;
+  Chunk ra, rw;
+  auto get = [&](const T* p, bool ok) {
+    Chunk c = Chunk(T(0));
+    if (ok) c = *reinterpret_cast<const Chunk*>(p);
+    return c;
+  };
+  auto fetch = [&](int k0) {
+    ra = get(a_src + k0, a_slot >= 0);
+    rw = get(w_src + k0, w_ok);
+  };
+  const int slot = sorted[p0 + 16 * wave + col];
+  f32x4 acc[4];  // [n tile]: lane holds C[m = col of m-tile `wave`][n = 4 grp + i]
+#pragma unroll
+  for (int i = 0; i < 4; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  fetch(0);
+  for (int k0 = 0; k0 < K; k0 += BK) {
+    __syncthreads();   // the previous slice has been read
+    *reinterpret_cast<Chunk*>(&As[s_row * LDK + s_k]) = ra;
+    *reinterpret_cast<Chunk*>(&Ws[s_row * LDK + s_k]) = rw;
+    __syncthreads();
+    if (k0 + BK < K) fetch(k0 + BK);
+    if constexpr (sizeof(T) == 2) {
+      const bf16x8 af = *reinterpret_cast<const bf16x8*>(&As[(16 * wave + col) * LDK + 8 * grp]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const bf16x8 wf = *reinterpret_cast<const bf16x8*>(&Ws[(16 * i + col) * LDK + 8 * grp]);
+        acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, af, acc[i], 0, 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < BK; ks += 16) {
+        const F af = *reinterpret_cast<const F*>(&As[(16 * wave + col) * LDK + ks + 4 * grp]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const F wf = *reinterpret_cast<const F*>(&Ws[(16 * i + col) * LDK + ks + 4 * grp]);
+          acc[i] = mma16(wf, af, acc[i]);
+        }
+      }
+    }
+  }
+  if (slot < 0) return;
+  const int64_t r = scatter ? slot : p0 + 16 * wave + col;
+  if (act == 2) {   // gate / up column pairs, as `store_gated`
+    auto rnd = [](float v) { return Elem<T>::ld(Elem<T>::st(v)); };
+#pragma unroll
+    for (int i2 = 0; i2 < 2; ++i2)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        if (nb + 32 * i2 + 16 + 4 * grp + q < N) {
+          const float g = rnd(acc[2 * i2][q]), u = rnd(acc[2 * i2 + 1][q]);
+          out[r * out_stride + (nb >> 1) + 16 * i2 + 4 * grp + q] = Elem<T>::st(rnd(g / (1.0f + expf(-g))) * u);
+        }
+      }
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int n = nb + 16 * i + 4 * grp + q;
+      if (n < N) {
+        float v = acc[i][q];
+        if (act == 1) { v = fmaxf(v, 0.f); v *= v; }
+        out[r * out_stride + n] = Elem<T>::st(v);
+      }
+    }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void combine_kernel(const T* __restrict__ y, const float* __restrict__ wts,
                                                       float* __restrict__ out, int W, int top) {
@@ -361,6 +454,18 @@ BCG_API int bcg_moe_gemm(const void* a, int64_t a_stride, const void* w, void* o
   const bool full = vec && K % 16 == 0;   // whole, aligned fragments only
   const int esz = is_f32 ? 4 : 2;
   if (K % 32 == 0 && (a_stride * esz) % 16 == 0 && (reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(w)) % 16 == 0) {
+    if (static_cast<int64_t>(n_tiles) * grid.y < 512 && (N + 63) / 64 <= 65535) {   // a small step: 64-column workgroups
+      const dim3 ngrid(n_tiles, (N + 63) / 64);
+      if (is_f32)
+        moe_gemm_lds_narrow_kernel<float><<<ngrid, 256, 0, s>>>(static_cast<const float*>(a), a_stride, static_cast<const float*>(w),
+                                                               static_cast<float*>(out), out_stride, static_cast<const int*>(sorted),
+                                                               static_cast<const int*>(tile_expert), N, K, top, gather, scatter, act);
+      else
+        moe_gemm_lds_narrow_kernel<bf16_t><<<ngrid, 256, 0, s>>>(static_cast<const bf16_t*>(a), a_stride, static_cast<const bf16_t*>(w),
+                                                                static_cast<bf16_t*>(out), out_stride, static_cast<const int*>(sorted),
+                                                                static_cast<const int*>(tile_expert), N, K, top, gather, scatter, act);
+      return BCG_CHECK_LAUNCH();
+    }
     if (is_f32)
       moe_gemm_lds_kernel<float><<<grid, 256, 0, s>>>(static_cast<const float*>(a), a_stride, static_cast<const float*>(w),
                                                      static_cast<float*>(out), out_stride, static_cast<const int*>(sorted),
