@@ -199,7 +199,7 @@ class InferenceEngine:
         self.ops = get_ops(self.backend)
 
         model_dir = args.weights if args.weights not in ("random", "auto") else None
-        if model_dir and not os.path.exists(os.path.join(model_dir, "tokenizer.json")) and cfg.family in ("mofidra", "padadra", "mabivik"):
+        if model_dir and not os.path.exists(os.path.join(model_dir, "tokenizer.json")) and cfg.family in ("mofidra", "padadra", "mabivik", "sitidra"):
             from .tokenizer import IdTokenizer
             self.tokenizer = IdTokenizer(cfg.vocab_size)  # a checkpoint of weights only: prompts are token ids
         else:

@@ -11,6 +11,9 @@ def model_class(family: str):
     if family == "mabivik":
         from .mabivik import MabivikModel
         return MabivikModel
+    if family == "sitidra":
+        from .sitidra import SitidraModel
+        return SitidraModel
     from .transformer import DecoderModel
     return DecoderModel
 

@@ -576,6 +576,165 @@ class MabivikConfig:
         return n
 
 
+@dataclass(frozen=True)
+class ChunkAttentionSpec:
+    """Softmax attention with GQA, rotate-half rotary on the first ``rot_dims`` features of every
+    q / k head (0 = none), q and k divided by their root mean square per head after the rotation,
+    a configured score scale, a chunk mask (``chunk`` > 0: position i sees j <= i only when
+    floor(i / chunk) = floor(j / chunk); 0 = plain causal), optional value mixing (``v_mix``: every
+    such layer but the first blends its values with the first one's values of the same token) and
+    one sigmoid output gate per head."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    chunk: int = 0
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    v_mix: bool = False
+
+
+@dataclass(frozen=True)
+class MatrixMemorySpec:
+    """Matrix memory with exponential gating (mLSTM): per head a ``dim x vdim`` memory, a
+    ``dim`` normaliser and a running maximum of the log gates; input and forget gate logits
+    are soft-capped at ``gate_cap``."""
+    heads: int
+    dim: int
+    vdim: int
+    gate_cap: float
+
+
+@dataclass(frozen=True)
+class ScoredRouterSpec:
+    """Mixture of gated experts whose router scores are sigmoids: ``top`` of ``experts`` experts of
+    width ``ff`` per token, chosen by score + correction among the ``keep`` best of ``groups``
+    groups of neighbouring experts; weights are the chosen scores over their sum, times ``scale``;
+    ``shared_ff`` > 0: an always-on expert of that width is added."""
+    ff: int
+    experts: int
+    top: int
+    groups: int = 1
+    keep: int = 1
+    scale: float = 1.0
+    shared_ff: int = 0
+
+
+@dataclass(frozen=True)
+class SitidraLayer:
+    type: str                    # "attention" | "mlstm"
+    mixer: object                # ChunkAttentionSpec | MatrixMemorySpec
+    mlp: Optional[ScoredRouterSpec]
+
+
+@dataclass(frozen=True)
+class SitidraConfig:
+    """Sitidra: pre-norm decoder (layer norms with a weight and no bias) over ``streams``
+    hyper-connection residual streams (0 = one plain residual stream), mixers of two kinds (chunked
+    softmax attention, matrix memory) in the order the config lists, mixture-of-experts
+    feed-forwards with sigmoid-scored grouped routing and a shared expert, soft-capped logits
+    (``logit_softcap`` 0 = none).  Everything is read from the model directory's config.json."""
+    name: str
+    hidden_size: int
+    vocab_size: int
+    layers: tuple
+    streams: int = 0
+    rms_eps: float = 1e-6
+    logit_softcap: float = 0.0
+    family: str = "sitidra"
+    max_position: int = 1 << 20
+    tie_embeddings: bool = False
+
+    @classmethod
+    def from_dict(cls, c: dict, name: str = "sitidra") -> "SitidraConfig":
+        layers = []
+        for entry in c["layers"]:
+            m, kind = entry["mixer"], entry["type"]
+            if kind == "attention":
+                rot = m.get("rot") or {}
+                mixer = ChunkAttentionSpec(
+                    heads=int(m["heads"]), kv_heads=int(m.get("kv_heads") or m["heads"]), dim=int(m["dim"]),
+                    vdim=int(m.get("vdim") or m["dim"]), scale=float(m["scale"]), chunk=int((m.get("mask") or {}).get("size", 0)),
+                    rot_dims=int(rot.get("dims", 0)), rot_base=float(rot.get("base", 10000.0)), v_mix=bool(m.get("v_mix", False)))
+                if mixer.heads % mixer.kv_heads or mixer.rot_dims % 2 or mixer.rot_dims > mixer.dim or mixer.chunk < 0:
+                    raise ValueError("Sitidra: heads must be a multiple of kv_heads, rot.dims even and <= dim")
+            elif kind == "mlstm":
+                mixer = MatrixMemorySpec(int(m["heads"]), int(m["dim"]), int(m.get("vdim") or m["dim"]), float(m["gate_cap"]))
+                if not mixer.gate_cap > 0:
+                    raise ValueError("Sitidra: gate_cap must be positive")
+            else:
+                raise ValueError(f"Sitidra: unknown layer type {kind!r}")
+            f = entry.get("mlp")
+            mlp = None
+            if f is not None:
+                if f.get("kind", "moe") != "moe":
+                    raise ValueError(f"Sitidra: unknown feed-forward kind {f['kind']!r}")
+                r = f["router"]
+                grp = r.get("groups") or {}
+                mlp = ScoredRouterSpec(ff=int(f["expert"]["ff"]), experts=int(r["experts"]), top=int(r["top"]),
+                                       groups=int(grp.get("count", 1)), keep=int(grp.get("keep", grp.get("count", 1))),
+                                       scale=float(r.get("scale", 1.0)), shared_ff=int((f.get("shared") or {}).get("ff", 0)))
+                if (not 1 <= mlp.top <= mlp.experts or mlp.groups < 1 or mlp.experts % mlp.groups
+                        or not 1 <= mlp.keep <= mlp.groups or mlp.top > mlp.keep * (mlp.experts // mlp.groups)):
+                    raise ValueError("Sitidra: router.top in [1, experts], equal groups, top experts within the kept groups")
+            layers.append(SitidraLayer(kind, mixer, mlp))
+        mixers = [l.mixer for l in layers if l.type == "attention" and l.mixer.v_mix]
+        if any((a.kv_heads, a.vdim) != (mixers[0].kv_heads, mixers[0].vdim) for a in mixers):
+            raise ValueError("Sitidra: layers that mix values need values of one shape")
+        return cls(name=name, hidden_size=int(c["width"]), vocab_size=int(c["vocab"]), layers=tuple(layers),
+                   streams=int(c.get("streams") or 0), rms_eps=float(c["norm"]["eps"]),
+                   logit_softcap=float(c.get("logit_softcap") or 0.0))
+
+    def to_dict(self) -> dict:
+        """The config.json form (inverse of `from_dict`)."""
+        out = []
+        for l in self.layers:
+            m = l.mixer
+            if l.type == "attention":
+                mixer = {"heads": m.heads, "kv_heads": m.kv_heads, "dim": m.dim, "vdim": m.vdim, "scale": m.scale}
+                if m.rot_dims:
+                    mixer["rot"] = {"dims": m.rot_dims, "base": m.rot_base}
+                if m.chunk:
+                    mixer["mask"] = {"size": m.chunk}
+                if m.v_mix:
+                    mixer["v_mix"] = True
+            else:
+                mixer = {"heads": m.heads, "dim": m.dim, "vdim": m.vdim, "gate_cap": m.gate_cap}
+            mlp = None
+            if l.mlp is not None:
+                f = l.mlp
+                mlp = {"kind": "moe", "expert": {"ff": f.ff},
+                       "router": {"experts": f.experts, "top": f.top, "scale": f.scale,
+                                  "groups": {"count": f.groups, "keep": f.keep}}}
+                if f.shared_ff:
+                    mlp["shared"] = {"ff": f.shared_ff}
+            out.append({"type": l.type, "mixer": mixer, "mlp": mlp})
+        d = {"architecture": "Sitidra", "width": self.hidden_size, "vocab": self.vocab_size, "norm": {"eps": self.rms_eps},
+             "layers": out}
+        if self.streams:
+            d["streams"] = self.streams
+        if self.logit_softcap:
+            d["logit_softcap"] = self.logit_softcap
+        return d
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    def num_params(self) -> int:
+        W, n = self.hidden_size, 2 * self.vocab_size * self.hidden_size + self.hidden_size
+        for l in self.layers:
+            m = l.mixer
+            if l.type == "attention":
+                n += W * (m.heads * m.dim + m.kv_heads * (m.dim + m.vdim) + m.heads) + W * m.heads * m.vdim
+            else:
+                n += W * (2 * m.heads * m.dim + 3 * m.heads * m.vdim + 2 * m.heads)
+            if l.mlp is not None:
+                n += l.mlp.experts * (3 * W * l.mlp.ff + W) + 3 * W * l.mlp.shared_ff
+        return n
+
+
 PRESETS = {
     "Qwen/Qwen3-8B": ModelConfig("Qwen/Qwen3-8B", "qwen3", 4096, 36, 32, 8, 128, 12288, 151936,
                                  qk_norm=True, max_position=40960),
@@ -615,6 +774,8 @@ def from_hf_config(path: str, name: Optional[str] = None):
         return PadadraConfig.from_dict(c, name or path)
     if str(c.get("architecture", "")).lower() == "mabivik":
         return MabivikConfig.from_dict(c, name or path)
+    if str(c.get("architecture", "")).lower() == "sitidra":
+        return SitidraConfig.from_dict(c, name or path)
     arch = (c.get("model_type") or "").lower()
     family = "qwen3" if arch == "qwen3" else ("qwen2" if arch == "qwen2" else "mistral")
     heads = c["num_attention_heads"]

@@ -23,14 +23,15 @@ def _torch_ops() -> SimpleNamespace:
                 tile_rows=64):
         return _ref.paged_attention(q, k_cache, v_cache, layer, block_tables, q_start, seq_lens, scale)
 
-    def multimap_attention(q, k_cache, v_cache, meta, scale, maps, lam, head_eps, out_scale, vdim, window=0, sink=None):
+    def multimap_attention(q, k_cache, v_cache, meta, scale, maps, lam, head_eps, out_scale, vdim, window=0, sink=None,
+                           chunk=0):
         # tiles / single-row lists only tell the HIP kernels how to walk the batch
         q_start = meta.q_start
         if q_start is None:  # decode: one row per sequence
             q_start = torch.arange(q.shape[0] + 1, dtype=torch.int32, device=q.device)
         lens = meta.seq_lens if meta.attn_seq_lens is None else meta.attn_seq_lens
         return _ref.multimap_attention(q, k_cache, v_cache, meta.block_tables, q_start, lens, scale, maps,
-                                       lam, head_eps, out_scale, vdim, window, sink)
+                                       lam, head_eps, out_scale, vdim, window, sink, chunk)
 
     return SimpleNamespace(
         name="torch",
@@ -63,6 +64,13 @@ def _torch_ops() -> SimpleNamespace:
         gated_group_norm=_ref.gated_group_norm,
         moe_table_route=_ref.moe_table_route,
         gelu_gather_mul=_ref.gelu_gather_mul,
+        gated_act=_ref.gated_act,
+        hyper_embed_norm=_ref.hyper_embed_norm,
+        hyper_update_norm=_ref.hyper_update_norm,
+        rope_norm_kv_write=_ref.rope_norm_kv_write,
+        exp_gate_prepare=_ref.exp_gate_prepare,
+        moe_route_scored=_ref.moe_route_scored,
+        softcap=_ref.softcap,
         linear=torch.nn.functional.linear,
         rmsnorm=_ref.rmsnorm,
         add_rmsnorm=_ref.add_rmsnorm,

@@ -102,7 +102,7 @@ def load_library(path: str = None) -> ctypes.CDLL:
         "bcg_multimap_split_keys": [],
         "bcg_multimap_attention": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                                    c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
-                                   c_float, c_float, c_float, c_float, c_int, c_int, c_int, c_void_p, c_void_p],
+                                   c_float, c_float, c_float, c_float, c_int, c_int, c_int, c_int, c_void_p, c_void_p],
         "bcg_embed_hashed_bigram": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_float,
                                     c_void_p, c_int, c_int, c_int, c_float, c_float, c_float, c_void_p, c_void_p, c_void_p,
                                     c_int, c_int, c_int, c_int, c_int, c_void_p],
@@ -119,9 +119,22 @@ def load_library(path: str = None) -> ctypes.CDLL:
         "bcg_delta_prepare": [c_void_p, c_int64, c_void_p, c_int64, c_int, c_void_p, c_int64, c_int, c_void_p, c_void_p,
                               c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
         "bcg_gated_state_scan": [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
-                                 c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
-        "bcg_head_norm_gate": [c_void_p, c_void_p, c_float, c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                               c_void_p],
+                                 c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "bcg_head_norm_gate": [c_void_p, c_void_p, c_float, c_void_p, c_int64, c_void_p, c_int, c_int, c_int, c_int, c_void_p,
+                               c_int, c_int, c_void_p],
+        "bcg_hyper_embed_norm": [c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int, c_int,
+                                 c_int, c_int, c_void_p],
+        "bcg_hyper_update_norm": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p,
+                                  c_int, c_int, c_int, c_int, c_void_p],
+        "bcg_rope_norm_kv_write": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_float, c_void_p, c_int64,
+                                   c_float, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                   c_int, c_void_p],
+        "bcg_exp_gate_prepare": [c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_float,
+                                 c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                                 c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+        "bcg_softcap": [c_void_p, c_int64, c_float, c_void_p],
+        "bcg_moe_route_scored": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                 c_float, c_int, c_void_p],
         "bcg_embed_scale_dyt": [c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                 c_int, c_int, c_void_p],
         "bcg_residual_post_norm": [c_void_p, c_void_p, c_int, c_int, c_float, c_void_p, c_void_p, c_float, c_int, c_float,
@@ -131,7 +144,7 @@ def load_library(path: str = None) -> ctypes.CDLL:
                                 c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
         "bcg_rope_half_tail": [c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_float, c_int,
                                c_int, c_int, c_void_p],
-        "bcg_gate_mul": [c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_void_p],
+        "bcg_gate_mul": [c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p],
         "bcg_gated_act": [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p],
         "bcg_ssm_prepare": [c_void_p, c_int64, c_int, c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                             c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
@@ -613,6 +626,8 @@ def hip_ops() -> SimpleNamespace:
     extra.update(seqstate_ops(lib))
     from .seqlatent import seqlatent_ops
     extra.update(seqlatent_ops(lib))
+    from .seqhyper import seqhyper_ops
+    extra.update(seqhyper_ops(lib))
 
     return SimpleNamespace(name="hip", **extra, rmsnorm_fp8=rmsnorm_fp8, embed_rmsnorm_fp8=embed_rmsnorm_fp8,
                            linear_fp8_residual=linear_fp8_residual, linear=linear, linear_silu=linear_silu, linear_residual=linear_residual,

@@ -405,12 +405,14 @@ def rope_multi_kv_write(qkv, positions, slots, n_q: int, n_kv: int, maps: int, d
 
 
 def multimap_attention(q, k_cache, v_cache, block_tables, q_start, seq_lens, scale: float, maps: int,
-                       lam: float, head_eps: float, out_scale: float, vdim: int, window: int = 0, sink=None):
+                       lam: float, head_eps: float, out_scale: float, vdim: int, window: int = 0, sink=None,
+                       chunk: int = 0):
     """Causal GQA attention with ``maps`` softmax maps per head over shared values:
     ``o = a_0 - lam * a_1`` (maps = 2; maps = 1: ``a_0``), then per head
     ``o / sqrt(mean(o^2) + head_eps) * out_scale`` (``head_eps < 0``: only the scale).
     Sequence b's query rows ``q_start[b]:q_start[b+1]`` are its last positions.  ``window`` > 0:
-    position i sees only j with i - j < window.  ``sink`` fp32 [n_q]: the softmax denominator of
+    position i sees only j with i - j < window.  ``chunk`` > 0: position i sees only j of its own
+    chunk, floor(j / chunk) = floor(i / chunk), chunks counted from position 0.  ``sink`` fp32 [n_q]: the softmax denominator of
     head h also holds ``exp(sink[h])`` (no key, no value, not scaled).  Returns
     ``[T, n_q * vdim]``; fp32 math."""
     T, n_q, qd = q.shape
@@ -435,6 +437,8 @@ def multimap_attention(q, k_cache, v_cache, block_tables, q_start, seq_lens, sca
         hidden = kpos > qpos
         if window > 0:
             hidden = hidden | (kpos < qpos - window + 1)
+        if chunk > 0:
+            hidden = hidden | (kpos < qpos - qpos % chunk)
         o = None
         for m in range(maps):
             sc = torch.matmul(qb[..., m * dim:(m + 1) * dim], k[..., m * dim:(m + 1) * dim].transpose(1, 2)) * scale
@@ -692,7 +696,7 @@ def delta_prepare(c, y, off_beta: int, a, a_log, dt_bias, heads: int, kv_heads: 
     return q, k, g, beta
 
 
-def gated_state_scan(q, k, g, v, beta, meta, state, delta: bool):
+def gated_state_scan(q, k, g, v, beta, meta, state, delta: bool, unit_last: bool = False):
     """Per head a ``dim x vdim`` fp32 state S, token after token:
 
         S <- diag(g_t) S;   u = v_t  (times beta_t when given)   (delta False)
@@ -702,11 +706,16 @@ def gated_state_scan(q, k, g, v, beta, meta, state, delta: bool):
     q / k [T, Gq, dim] fp32 (head h reads q / k head h // (H / Gq)), g fp32 [T, H, dim] (a decay
     per key channel) or [T, H, 1] (one per head), v [T, H vdim], beta [T, H] fp32 or None;
     ``state`` [rows, H, dim, vdim] fp32 is read (unless the segment starts at position 0) and left
-    at the segment's last token.  Returns fp32 o [T, H, vdim]."""
+    at the segment's last token.  ``unit_last`` (without the delta rule): v is [T, H (vdim - 1)] and the
+    state's last column reads a value of 1 for every token, so it accumulates the written keys alone
+    (a normaliser beside the memory); o's last column is then its product with q.  Returns fp32 o [T, H, vdim]."""
     T, H = g.shape[:2]
     vdim = state.shape[3]
     per = H // q.shape[1]
-    vf = v.float().reshape(T, H, vdim)
+    if unit_last:
+        vf = torch.cat([v.float().reshape(T, H, vdim - 1), torch.ones(T, H, 1, device=v.device)], -1)
+    else:
+        vf = v.float().reshape(T, H, vdim)
     qh, kh = q.repeat_interleave(per, 1), k.repeat_interleave(per, 1)
     out = torch.zeros(T, H, vdim, dtype=torch.float32, device=g.device)
     qs = meta.q_start.tolist()
@@ -730,12 +739,15 @@ def gated_state_scan(q, k, g, v, beta, meta, state, delta: bool):
     return out
 
 
-def head_norm_gate(o, w, eps: float, gate, out_dtype, gate_act: str = "sigmoid"):
-    """o fp32 [T, H, vdim]: every head divided by its root mean square, times ``w`` [vdim], times
-    ``sigmoid(gate)`` or ``silu(gate)`` (gate [T, H vdim] logits or None; ``gate_act``); returns
-    [T, H vdim] in ``out_dtype``."""
+def head_norm_gate(o, w, eps: float, gate, out_dtype, gate_act: str = "sigmoid", floor=None):
+    """o fp32 [T, H, vdim]: every head divided by its root mean square, times ``w`` ([vdim], or
+    [H vdim]: a weight per head), times ``sigmoid(gate)`` or ``silu(gate)`` (gate [T, H vdim] logits or
+    None; ``gate_act``); returns [T, H vdim] in ``out_dtype``.  ``floor`` fp32 [T, H]: o has one more
+    column, a normaliser, and the head is first divided by ``max(|normaliser|, floor) + 1e-6``."""
+    if floor is not None:
+        o = o[..., :-1] / (torch.maximum(o[..., -1].abs(), floor.float()) + 1e-6)[..., None]
     T, H, vdim = o.shape
-    y = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+    y = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * w.float().reshape(-1, vdim)
     if gate is not None:
         z = gate.float().reshape(T, H, vdim)
         y = y * (torch.sigmoid(z) if gate_act == "sigmoid" else z * torch.sigmoid(z))
@@ -851,9 +863,10 @@ def head_linear(x3, w, out3=None):
     return out3
 
 
-def gate_mul(x, gate, kind: str):
-    """``x * sigmoid(gate)`` or ``x * silu(gate)`` (fp32, rounded once); gate [T, n] with any row stride."""
-    z = gate.float()
+def gate_mul(x, gate, kind: str, group: int = 1):
+    """``x * sigmoid(gate)`` or ``x * silu(gate)`` (fp32, rounded once); gate [T, n / group] with any
+    row stride: one gate column serves ``group`` neighbouring columns of x (one gate per head)."""
+    z = gate.float().repeat_interleave(group, 1) if group > 1 else gate.float()
     return (x.float() * (torch.sigmoid(z) if kind == "sigmoid" else z * torch.sigmoid(z))).to(x.dtype)
 
 
@@ -892,3 +905,135 @@ def gelu_gather_mul(z, tokens, table, off: int):
     """``gelu_tanh(z) * table[token, off : off + n]`` for z [T, n] (fp32 math, rounded once)."""
     e = table.index_select(0, tokens.long())[:, off:off + z.shape[1]].float()
     return (act_fn(z.float(), "gelu_tanh") * e).to(z.dtype)
+
+
+def gated_act(both):
+    """``silu(both[:, :n]) * both[:, n:]`` for a stacked [gate | up] projection [rows, 2 n]; the
+    activation is rounded like a projection's output before the product."""
+    n = both.shape[1] // 2
+    return (act_fn(both[:, :n], "silu").float() * both[:, n:].float()).to(both.dtype)
+
+
+# ------------------------------------------------------------------ hyper-connection streams, layer norms, unit-norm rotary
+# heads with value mixing, exponential-gate matrix memory, sigmoid-scored grouped routing (models/sitidra.py)
+#
+# The residual is S streams X [T, S, W] fp32.  A sublayer reads ``u = sum_s read[s] X[s]`` through a
+# layer norm and its output y is written back as ``X'[t] = sum_s mix[s, t] X[s] + out[t] y``, all
+# streams from the old ones.  S = 1 with read = mix = out = 1 is the plain residual sum.
+
+def layer_norm32(u, w, eps: float, out_dtype):
+    """fp32 ``(u - mean) / sqrt(var + eps) * w`` (biased variance, no bias), rounded once."""
+    uf = u.float()
+    d = uf - uf.mean(-1, keepdim=True)
+    return (d * torch.rsqrt(d.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(out_dtype)
+
+
+def hyper_embed_norm(tokens, table, streams: int, read_w, norm_w, eps: float, out_dtype):
+    """(X fp32 [T, streams, W] with every stream = table[token], layer norm of ``sum_s read_w[s] X[s]``)."""
+    x = table.index_select(0, tokens.long()).float()
+    X = x[:, None, :].repeat(1, streams, 1).contiguous()
+    return X, layer_norm32(torch.einsum("s,nsw->nw", read_w.float(), X), norm_w, eps, out_dtype)
+
+
+def hyper_update_norm(X, parts, mix, out_w, read_w, norm_w, eps: float, out_dtype):
+    """In place ``X[:, t] <- sum_s mix[s, t] X[:, s] + out_w[t] y`` with y the fp32 sum of ``parts``
+    (``mix`` None: X stays); returns the layer norm of ``sum_s read_w[s] X[:, s]`` (``read_w`` None: None)."""
+    if mix is not None:
+        y = None
+        for p in parts:
+            y = p.float() if y is None else y + p.float()
+        new = torch.einsum("sd,nsw->ndw", mix.float(), X)
+        if y is not None:
+            new = new + out_w.float()[None, :, None] * y[:, None, :]
+        X.copy_(new)
+    if read_w is None:
+        return None
+    return layer_norm32(torch.einsum("s,nsw->nw", read_w.float(), X), norm_w, eps, out_dtype)
+
+
+def rope_norm_kv_write(qkv, positions, slots, n_q: int, n_kv: int, dim: int, vdim: int, inv_freq, qk_eps: float,
+                       v_first, lam: float, k_cache, v_cache):
+    """Split a fused projection row ``[q | k | v | anything]``; rotate the first ``2 * len(inv_freq)``
+    features of every q / k head (feature i pairs with i + rot/2; angle = position * inv_freq[i], fp32);
+    divide every head by its root mean square over ``dim`` (``qk_eps`` < 0: not); blend the values,
+    ``v <- (1 - lam) v + lam v_first`` (``v_first`` [T, n_kv vdim], any row stride; None: v as it is);
+    scatter K / V into the paged cache.  Returns q ``[T, n_q, dim]`` in the activation dtype."""
+    T = qkv.shape[0]
+    qw, kw = n_q * dim, n_kv * dim
+    q = qkv[:, :qw].float().reshape(T, n_q, dim)
+    k = qkv[:, qw:qw + kw].float().reshape(T, n_kv, dim)
+    v = qkv[:, qw + kw:qw + kw + n_kv * vdim].float()
+    half = inv_freq.numel()
+    if half:
+        ang = positions.float()[:, None] * inv_freq.float()[None, :]
+        cos, sin = ang.cos()[:, None, :], ang.sin()[:, None, :]
+
+        def rot(x):
+            a, b, rest = x[..., :half], x[..., half:2 * half], x[..., 2 * half:]
+            return torch.cat([a * cos - b * sin, b * cos + a * sin, rest], dim=-1)
+        q, k = rot(q), rot(k)
+    if qk_eps >= 0:
+        q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + qk_eps)
+        k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + qk_eps)
+    if v_first is not None:
+        v = (1.0 - lam) * v + lam * v_first.float()
+    bs = k_cache.shape[2]
+    blk, off = (slots // bs).long(), (slots % bs).long()
+    k_cache[blk, :, off] = k.to(k_cache.dtype)
+    v_cache[blk, :, :, off] = v.reshape(T, n_kv, vdim).to(v_cache.dtype)
+    return q.to(qkv.dtype)
+
+
+def exp_gate_prepare(y, off_q: int, off_k: int, off_i: int, off_f: int, i_bias, f_bias, cap: float, q_scale: float,
+                     heads: int, dim: int, meta, m_state):
+    """Gates of a matrix memory from the fused projection ``y``: per head the log input gate
+    ``i = cap tanh((y_i + b_i) / cap)`` and the log forget gate ``f = logsigmoid(cap tanh((y_f + b_f) / cap))``,
+    the running maximum ``m_t = max(f_t + m_(t-1), i_t)`` (``m_state`` fp32 [rows, heads], read unless
+    the segment starts at position 0 -- it then starts at 0 -- and left at the segment's last token).
+    Returns fp32 (q_scale * q [T, heads, dim], k [T, heads, dim], decay ``exp(f_t + m_(t-1) - m_t)``
+    [T, heads, 1], write scale ``exp(i_t - m_t)`` [T, heads], floor ``exp(-m_t)`` [T, heads])."""
+    T, n = y.shape[0], heads * dim
+    q = (y[:, off_q:off_q + n].float() * q_scale).reshape(T, heads, dim).contiguous()
+    k = y[:, off_k:off_k + n].float().reshape(T, heads, dim).contiguous()
+    gi = cap * torch.tanh((y[:, off_i:off_i + heads].float() + i_bias.float()) / cap)
+    gf = torch.nn.functional.logsigmoid(cap * torch.tanh((y[:, off_f:off_f + heads].float() + f_bias.float()) / cap))
+    decay = torch.empty(T, heads, dtype=torch.float32, device=y.device)
+    write, floor = torch.empty_like(decay), torch.empty_like(decay)
+    qs, rows, pos = meta.q_start.tolist(), meta.state_rows.tolist(), meta.positions.tolist()
+    for b in range(len(rows)):
+        s, e = qs[b], qs[b + 1]
+        if e <= s:
+            continue
+        m = m_state[rows[b]].clone() if pos[s] > 0 else torch.zeros(heads, dtype=torch.float32, device=y.device)
+        for t in range(s, e):
+            new = torch.maximum(gf[t] + m, gi[t])
+            decay[t], write[t], floor[t] = torch.exp(gf[t] + m - new), torch.exp(gi[t] - new), torch.exp(-new)
+            m = new
+        m_state[rows[b]] = m
+    return q, k, decay[:, :, None].contiguous(), write, floor
+
+
+def moe_route_scored(h, router_w, corr, top: int, groups: int, keep: int, scale: float):
+    """fp32 router with sigmoid scores ``s = sigmoid(W h)``.  The ``top`` experts with the largest choice
+    score ``s + corr`` (ties: lowest index) among the ``keep`` best of ``groups`` equal groups of neighbouring
+    experts (a group's score: the sum of its two largest choice scores; ties: lowest group); the others
+    cannot be chosen.  Weights: the chosen ``s`` over their sum (+ 1e-20), times ``scale``.  Returns
+    (expert ids int32 [T, top], weights fp32 [T, top])."""
+    sc = torch.sigmoid(h.float() @ router_w.float().t())
+    choice = sc if corr is None else sc + corr.float()
+    T, E = choice.shape
+    if groups > 1 and keep < groups:
+        per = E // groups
+        g = choice.reshape(T, groups, per)
+        gs = g.topk(min(2, per), dim=-1).values.sum(-1)
+        order = torch.sort(gs, dim=-1, descending=True, stable=True).indices[:, :keep]
+        allowed = torch.zeros(T, groups, dtype=torch.bool, device=h.device).scatter_(1, order, True)
+        choice = g.masked_fill(~allowed[:, :, None], float("-inf")).reshape(T, E)
+    idx = torch.sort(choice, dim=-1, descending=True, stable=True).indices[:, :top]
+    w = sc.gather(1, idx)
+    return idx.to(torch.int32), w / (w.sum(-1, keepdim=True) + 1e-20) * scale
+
+
+def softcap(logits, cap: float):
+    """``cap tanh(logits / cap)`` on fp32 logits, in place."""
+    return logits.copy_(cap * torch.tanh(logits / cap))

@@ -108,12 +108,19 @@ def seqlatent_ops(lib):
             torch.bmm(x3.transpose(0, 1), w.transpose(1, 2), out=out3.transpose(0, 1))
         return out3
 
-    def gate_mul(x, gate, kind):
-        _req(x.dim() == 2 and x.is_contiguous() and gate.shape == x.shape and gate.stride(1) == 1 and gate.dtype == x.dtype,
-             "gate_mul: x [T, n] contiguous, gate [T, n] with unit column stride")
+    def gate_mul(x, gate, kind, group=1):
+        _req(x.dim() == 2 and x.is_contiguous() and group >= 1 and gate.shape == (x.shape[0], x.shape[1] // group)
+             and x.shape[1] % group == 0 and gate.stride(1) == 1 and gate.dtype == x.dtype,
+             "gate_mul: x [T, n] contiguous, gate [T, n / group] with unit column stride")
         out = torch.empty_like(x)
         _check(lib.bcg_gate_mul(_p(x), _p(gate), gate.stride(0), _p(out), x.shape[0], x.shape[1], {"sigmoid": 0, "silu": 1}[kind],
-                                _act(x), _stream()), "gate_mul")
+                                group, _act(x), _stream()), "gate_mul")
+        return out
+
+    def gated_act(both):
+        _req(both.dim() == 2 and both.is_contiguous() and both.shape[1] % 2 == 0, "gated_act: [rows, 2 n] contiguous")
+        out = torch.empty(both.shape[0], both.shape[1] // 2, dtype=both.dtype, device=both.device)
+        _check(lib.bcg_gated_act(_p(both), _p(out), both.shape[0], both.shape[1] // 2, _act(both), _stream()), "gated_act")
         return out
 
     def ssm_prepare(c, off_b, y, off_dt, dt_bias, a_log, heads, groups, state):
@@ -164,4 +171,4 @@ def seqlatent_ops(lib):
     return dict(embed_scale_dyt=embed_scale_dyt, residual_post_norm=residual_post_norm, rmsnorm_cols=rmsnorm_cols,
                 latent_kv_write=latent_kv_write, rope_half_tail=rope_half_tail, head_linear=head_linear, gate_mul=gate_mul,
                 ssm_prepare=ssm_prepare, gated_group_norm=gated_group_norm, moe_table_route=moe_table_route,
-                gelu_gather_mul=gelu_gather_mul)
+                gelu_gather_mul=gelu_gather_mul, gated_act=gated_act)

@@ -137,10 +137,12 @@ def seqmix_ops(lib, linear):
         """Query rows per prefill tile (the tile table the engine builds) for these head sizes."""
         return 64  # four waves x 16 rows
 
-    def multimap_attention(q, k_cache, v_cache, meta, scale, maps, lam, head_eps, out_scale, vdim, window=0, sink=None):
+    def multimap_attention(q, k_cache, v_cache, meta, scale, maps, lam, head_eps, out_scale, vdim, window=0, sink=None,
+                           chunk=0):
         """Prefill tiles (``meta.tiles``) on the MFMA kernel, one-token rows (``meta.single``, or
-        every row of a decode step) on the split-KV kernel.  ``window`` / ``sink`` (one-map heads):
-        sliding window in keys, fp32 [H] sink logits of the softmax denominator."""
+        every row of a decode step) on the split-KV kernel.  ``window`` / ``chunk`` / ``sink``
+        (one-map heads): sliding window in keys, or a chunk mask (a query sees the keys of its own
+        ``chunk``-aligned block of positions only); fp32 [H] sink logits of the softmax denominator."""
         T, H, qd = q.shape
         _req(q.is_contiguous() and qd % maps == 0, "q [T, H, maps dim] contiguous")
         dim = qd // maps
@@ -156,16 +158,17 @@ def seqmix_ops(lib, linear):
         f32 = _act(q)
         tile_rows = meta.tile_rows if not meta.decode else 64
         _req(tile_rows == 64, "prefill tiles: 64 query rows")
-        window = int(window or 0)
-        _req(window >= 0 and (maps == 1 or (window == 0 and sink is None)), "window / sink: one-map heads")
+        window, chunk = int(window or 0), int(chunk or 0)
+        _req(window >= 0 and chunk >= 0 and not (window and chunk)
+             and (maps == 1 or (window == 0 and chunk == 0 and sink is None)), "window / chunk / sink: one-map heads, one mask")
         if sink is not None:
             _req(sink.dtype == torch.float32 and sink.numel() == H and sink.is_contiguous(), "sink fp32 [H]")
-        common = (H, G, maps, dim, vdim, BS, NB, scale, lam, head_eps, out_scale, tile_rows, f32, window, _p(sink), _stream())
+        common = (H, G, maps, dim, vdim, BS, NB, scale, lam, head_eps, out_scale, tile_rows, f32, window, chunk, _p(sink), _stream())
 
         def decode(work, n_items):
             n_splits = max(1, (bt.shape[1] * BS + split_keys - 1) // split_keys)
-            if window:  # splits are counted from the window's first: it touches this many at most
-                n_splits = min(n_splits, (window + split_keys - 1) // split_keys + 1)
+            if window or chunk:  # splits are counted from the window's (chunk's) first: it touches this many at most
+                n_splits = min(n_splits, (max(window, chunk) + split_keys - 1) // split_keys + 1)
             ws = torch.empty(n_items * H * n_splits * (2 * maps + maps * vdim), dtype=torch.float32, device=q.device)
             _check(lib.bcg_multimap_attention(1, _p(q), _p(k_cache), _p(v_cache), _p(bt), bt.shape[1], None, _p(lens),
                                               _p(work), n_items, _p(out), _p(ws), n_splits, *common), "multimap decode")
@@ -202,6 +205,20 @@ def seqmix_ops(lib, linear):
         _check(lib.bcg_moe_route(_p(h), _p(router_w), _p(router_b), _p(gate_w), _p(idx), _p(wts), _p(gate), T, W, E, top,
                                  _act(h), _stream()), "moe_route")
         return idx, wts, gate
+
+    def moe_route_scored(h, router_w, corr, top, groups, keep, scale):
+        T, W = h.shape
+        E = router_w.shape[0]
+        _req(h.is_contiguous() and router_w.dtype == torch.float32 and router_w.shape == (E, W) and router_w.is_contiguous()
+             and (corr is None or (corr.dtype == torch.float32 and corr.numel() == E and corr.is_contiguous()))
+             and 1 <= top <= E <= 256, "moe_route_scored: fp32 router [E, W], fp32 correction [E], E <= 256")
+        _req(groups >= 1 and E % groups == 0 and 1 <= keep <= groups and top <= keep * (E // groups),
+             "moe_route_scored: equal groups, `top` experts inside the kept groups")
+        idx = torch.empty(T, top, dtype=torch.int32, device=h.device)
+        wts = torch.empty(T, top, dtype=torch.float32, device=h.device)
+        _check(lib.bcg_moe_route_scored(_p(h), _p(router_w), _p(corr), _p(idx), _p(wts), T, W, E, top, groups, keep,
+                                        float(scale), _act(h), _stream()), "moe_route_scored")
+        return idx, wts
 
     def moe_pair_rows(gate, up):
         """The [2 ff, W] weight of one gated expert as `moe_experts` (kind "silu_gated") reads it:
@@ -256,4 +273,4 @@ def seqmix_ops(lib, linear):
                 rmsnorm32=rmsnorm32, act_fn=act_fn, rope_multi_kv_write=rope_multi_kv_write,
                 kv_from_logical=kv_from_logical, kv_to_logical=kv_to_logical,
                 multimap_attention=multimap_attention, multimap_tile_rows=multimap_tile_rows, moe_route=moe_route, moe_experts=moe_experts,
-                moe_pair_rows=moe_pair_rows)
+                moe_pair_rows=moe_pair_rows, moe_route_scored=moe_route_scored)

@@ -169,7 +169,7 @@ def seqstate_ops(lib):
                "delta_prepare")
         return q, k, g, beta
 
-    def gated_state_scan(q, k, g, v, beta, meta, state, delta):
+    def gated_state_scan(q, k, g, v, beta, meta, state, delta, unit_last=False):
         T, H, gd = g.shape
         _req(state.dim() == 4 and state.dtype == torch.float32 and state.is_contiguous() and state.shape[1] == H,
              "state fp32 [rows, H, dim, vdim]")
@@ -180,21 +180,27 @@ def seqstate_ops(lib):
         for t, name in ((q, "q"), (k, "k")):
             _req(t.dtype == torch.float32 and t.is_contiguous() and t.shape == (T, Gq, dim), f"{name} fp32 [T, Gq, dim]")
         _req(g.dtype == torch.float32 and g.is_contiguous() and H % Gq == 0 and 1 <= dim <= 256, "g fp32 [T, H, dim], dim <= 256")
-        _req(v.dim() == 2 and v.stride(1) == 1 and v.shape == (T, H * vdim), "v [T, H vdim], unit column stride")
+        v_head = vdim - 1 if unit_last else vdim   # the state's last column then reads ones, not v
+        _req(v.dim() == 2 and v.stride(1) == 1 and v.shape == (T, H * v_head), "v [T, H vdim], unit column stride")
         _req(beta is not None or not delta, "the delta rule needs beta")
+        _req(not unit_last or (not delta and vdim >= 2), "a unit last column: without the delta rule")
         if beta is not None:
             _req(beta.dtype == torch.float32 and beta.is_contiguous() and beta.shape == (T, H), "beta fp32 [T, H]")
         B = _segments(meta, T)
         out = torch.empty(T, H, vdim, dtype=torch.float32, device=g.device)
         _check(lib.bcg_gated_state_scan(_p(q), _p(k), _p(g), _p(v), v.stride(0), _p(beta), _p(meta.positions),
                                         _p(meta.q_start), _p(meta.state_rows), _p(state), state.shape[0], _p(out), B, H, Gq, dim,
-                                        vdim, gd, int(bool(delta)), _act(v), _stream()), "gated_state_scan")
+                                        vdim, gd, int(bool(delta)), int(bool(unit_last)), _act(v), _stream()), "gated_state_scan")
         return out
 
-    def head_norm_gate(o, w, eps, gate, out_dtype, gate_act="sigmoid"):
+    def head_norm_gate(o, w, eps, gate, out_dtype, gate_act="sigmoid", floor=None):
         _req(o.dim() == 3 and o.dtype == torch.float32 and o.is_contiguous(), "o fp32 [T, H, vdim]")
         T, H, vdim = o.shape
-        _f32(w, vdim, "head norm weight")
+        if floor is not None:   # o's last column is a normaliser
+            vdim -= 1
+            _req(vdim >= 1 and floor.dtype == torch.float32 and floor.shape == (T, H) and floor.is_contiguous(), "floor fp32 [T, H]")
+        _req(w.numel() in (vdim, H * vdim), "head norm weight [vdim] or [H vdim]")
+        _f32(w, w.numel(), "head norm weight")
         stride = 0
         if gate is not None:
             _req(gate.dim() == 2 and gate.stride(1) == 1 and gate.shape == (T, H * vdim) and gate.dtype == out_dtype,
@@ -202,7 +208,8 @@ def seqstate_ops(lib):
             stride = gate.stride(0)
         out = torch.empty(T, H * vdim, dtype=out_dtype, device=o.device)
         _check(lib.bcg_head_norm_gate(_p(o), _p(w), eps, _p(gate), stride, _p(out), T, H, vdim,
-                                      {"sigmoid": 0, "silu": 1}[gate_act], int(out_dtype == torch.float32), _stream()),
+                                      {"sigmoid": 0, "silu": 1}[gate_act], _p(floor), vdim if w.numel() != vdim else 0,
+                                      int(out_dtype == torch.float32), _stream()),
                "head_norm_gate")
         return out
 

@@ -26,9 +26,10 @@
 // decode_merge_kernel merges the splits and applies the map combination + head norm.
 //
 // Optional, for one-map heads: a sliding window (a query at position i sees keys j with
-// i - j < window) and a per-head sink, a learned logit that takes part in the softmax denominator
-// only (no key, no value, not scaled).  The key loop starts at the window's first 16-key tile;
-// decode splits are counted from the window's first split.
+// i - j < window) or a chunk mask (position i sees j <= i of its own chunk, floor(i / chunk) ==
+// floor(j / chunk), chunks counted from position 0), and a per-head sink, a learned logit that takes part in the softmax denominator
+// only (no key, no value, not scaled).  The key loop starts at the window's (chunk's) first 16-key
+// tile; decode splits are counted from the window's (chunk's) first split.
 #include <algorithm>
 
 #include "seqmix_common.h"
@@ -53,9 +54,17 @@ struct AttnArgs {
   float scale, lam, head_eps, out_scale;
   int vec_k, vec_v;         // rows of K / V^T are aligned for 4-element vector loads
   int window;               // > 0: keys below position - window + 1 are hidden
+  int chunk;                // > 0: keys below position - position % chunk are hidden (chunks count from position 0)
   const float* sink;        // [H] or null
   int swz;                  // fragment-major slabs (see the top of the file)
 };
+
+// First key that a query at position `pos` sees: the window's or the chunk's first, else 0.
+__device__ __forceinline__ int first_key(const AttnArgs& a, int pos) {
+  if (a.window > 0) return max(0, pos - a.window + 1);
+  if (a.chunk > 0) return pos - pos % a.chunk;
+  return 0;
+}
 
 // The key loop shared by both kernels: keys [k_begin, k_last] of one sequence for the 16 query
 // columns of a wave (column = a query row of one head, or a query head of one token).
@@ -269,8 +278,8 @@ __global__ __launch_bounds__(256, OCC) void prefill_kernel(AttnArgs a) {
     mx[0] = a.sink[h] * LOG2E;
     den[0] = 1.0f;
   }
-  const int lo = a.window > 0 ? pos - a.window + 1 : 0, lo_max = a.window > 0 ? pos_max - a.window + 1 : 0;
-  const int k_begin = a.window > 0 ? (max(0, pos_min - a.window + 1) & ~15) : 0;
+  const int lo = first_key(a, pos), lo_max = first_key(a, pos_max);   // (both masks: the first key grows with the position)
+  const int k_begin = first_key(a, pos_min) & ~15;
   attend_range<T, KC, VT, KT, PF, FULL, EXACT, NM>(a, g, qf, pos, pos_min, lo, lo_max, k_begin, pos_max,
                                         a.block_tables + static_cast<size_t>(seq) * a.max_blocks, acc, mx, den);
   // ---- combine the maps, unit norm over the head's value features, store ----
@@ -323,7 +332,7 @@ __global__ __launch_bounds__(64, OCC) void decode_mfma_kernel(AttnArgs a) {
   const int split = blockIdx.y, item = blockIdx.z;
   const int row = a.work ? a.work[2 * item] : item, seq = a.work ? a.work[2 * item + 1] : item;
   const int ctx = a.seq_lens[seq];
-  const int lo = a.window > 0 ? max(0, ctx - a.window) : 0;          // first visible key
+  const int lo = first_key(a, ctx - 1);                             // first visible key
   const int split_abs = lo / SPLIT_KEYS + split;                    // splits count from the window's first
   const int k_end = min(ctx, (split_abs + 1) * SPLIT_KEYS);
   const int k_begin = max(split_abs * SPLIT_KEYS, lo & ~15);
@@ -382,7 +391,7 @@ __global__ __launch_bounds__(64) void decode_merge_kernel(AttnArgs a) {
   const int lane = threadIdx.x, h = blockIdx.x, item = blockIdx.y;
   const int row = a.work ? a.work[2 * item] : item, seq = a.work ? a.work[2 * item + 1] : item;
   const int ctx = a.seq_lens[seq];
-  const int s_first = a.window > 0 ? max(0, ctx - a.window) / SPLIT_KEYS : 0;
+  const int s_first = first_key(a, ctx - 1) / SPLIT_KEYS;
   const int n = min(a.n_splits, (ctx + SPLIT_KEYS - 1) / SPLIT_KEYS - s_first);
   const float sink = a.sink != nullptr ? a.sink[h] * LOG2E : MAX_FLOOR;
   const int stride = 2 * a.maps + a.maps * a.vdim;
@@ -520,9 +529,11 @@ BCG_API int bcg_multimap_attention(int mode, const void* q, const void* k_cache,
                                    const void* block_tables, int max_blocks, const void* q_start, const void* seq_lens,
                                    const void* work, int n_work, void* out, void* ws, int n_splits, int H, int G, int maps,
                                    int dim, int vdim, int BS, int num_blocks, float scale, float lam, float head_eps,
-                                   float out_scale, int tile_rows, int is_f32, int window, const void* sink, void* stream) {
+                                   float out_scale, int tile_rows, int is_f32, int window, int chunk, const void* sink,
+                                   void* stream) {
   if (n_work <= 0) return 0;
-  if ((window > 0 || sink != nullptr) && maps != 1) return -2;
+  if ((window > 0 || chunk > 0 || sink != nullptr) && maps != 1) return -2;
+  if (window > 0 && chunk > 0) return -2;
   if (maps < 1 || maps > 2 || dim > (maps == 1 ? 512 : 128) || vdim > 256 || BS % 16 || H % G || n_work > 65535 * 16) return -2;
   AttnArgs a;
   a.q = q; a.k_cache = k_cache; a.v_cache = v_cache;
@@ -535,7 +546,7 @@ BCG_API int bcg_multimap_attention(int mode, const void* q, const void* k_cache,
   a.vec_k = ((maps * dim) % 4 == 0) ? 1 : 0;
   a.vec_v = 1;  // BS % 16 == 0: every 4-key group of a V^T row is aligned
   a.swz = a.vec_k;
-  a.window = window; a.sink = static_cast<const float*>(sink);
+  a.window = window; a.chunk = chunk; a.sink = static_cast<const float*>(sink);
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (mode == 0) return is_f32 ? launch_prefill<float>(a, n_work, tile_rows, s) : launch_prefill<bf16_t>(a, n_work, tile_rows, s);
   if (n_splits < 1 || H > 65535 || n_splits > 65535 || n_work > 65535) return -2;

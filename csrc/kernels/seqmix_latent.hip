@@ -236,15 +236,16 @@ __global__ __launch_bounds__(NT) void rope_half_tail_kernel(const T* __restrict_
   }
 }
 
-// out = x * sigmoid(gate) (kind 0) or x * silu(gate) (kind 1); gate rows have their own stride.
+// out = x * sigmoid(gate) (kind 0) or x * silu(gate) (kind 1); gate rows have their own stride and
+// one gate column serves `group` neighbouring columns of x (group = a head's width: one gate per head).
 template <typename T>
 __global__ __launch_bounds__(NT) void gate_mul_kernel(const T* __restrict__ x, const T* __restrict__ gate, int64_t gate_stride,
-                                                      T* __restrict__ out, int64_t rows, int n, int kind) {
+                                                      T* __restrict__ out, int64_t rows, int n, int kind, int group) {
   const int64_t total = rows * n;
   for (int64_t e = static_cast<int64_t>(blockIdx.x) * NT + threadIdx.x; e < total; e += static_cast<int64_t>(gridDim.x) * NT) {
     const int64_t r = e / n;
     const int c = static_cast<int>(e - r * n);
-    const float g = Elem<T>::ld(gate[r * gate_stride + c]);
+    const float g = Elem<T>::ld(gate[r * gate_stride + c / group]);
     out[e] = Elem<T>::st(Elem<T>::ld(x[e]) * (kind == 0 ? sigmoidf_(g) : siluf_(g)));
   }
 }
@@ -422,13 +423,14 @@ BCG_API int bcg_rope_half_tail(const void* src, int Ds, int src_off, void* dst, 
 }
 
 BCG_API int bcg_gate_mul(const void* x, const void* gate, int64_t gate_stride, void* out, int64_t rows, int n, int kind,
-                         int is_f32, void* stream) {
+                         int group, int is_f32, void* stream) {
   if (rows <= 0 || n <= 0) return 0;
+  if (group < 1 || n % group) return -2;
   hipStream_t s = static_cast<hipStream_t>(stream);
   BCG_BY_TYPE((gate_mul_kernel<float><<<ew_grid(rows * n), NT, 0, s>>>(static_cast<const float*>(x), static_cast<const float*>(gate), gate_stride,
-                                                                      static_cast<float*>(out), rows, n, kind)),
+                                                                      static_cast<float*>(out), rows, n, kind, group)),
               (gate_mul_kernel<bf16_t><<<ew_grid(rows * n), NT, 0, s>>>(static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(gate), gate_stride,
-                                                                       static_cast<bf16_t*>(out), rows, n, kind)));
+                                                                       static_cast<bf16_t*>(out), rows, n, kind, group)));
   return BCG_CHECK_LAUNCH();
 }
 

@@ -1,7 +1,10 @@
 // Mixture-of-experts feed-forward with device-side routing (no host synchronisation):
 //
 //   route   : fp32 logits z = R h + b, the `top` largest (ties: lowest index), softmax over
-//             those only; also the fp32 logit of the always-on expert's gate
+//             those only; also the fp32 logit of the always-on expert's gate.  Scored form:
+//             s = sigmoid(z); the choice goes by s + correction, limited to the `keep` best of
+//             `groups` equal groups of neighbouring experts (a group's score: the sum of its two
+//             largest choice scores); weights s / (sum of the chosen s + 1e-20) * scale
 //   align   : slots (token, j) bucketed by expert into tile-aligned position ranges
 //   gemm    : per position tile (one expert) C = A W_e^T on 16 x 16 MFMAs; "up" gathers token
 //             rows and applies the activation, "down" scatters rows back to their slots
@@ -22,8 +25,9 @@ template <typename T>
 __global__ __launch_bounds__(256) void route_kernel(const T* __restrict__ h, const float* __restrict__ rw,
                                                     const float* __restrict__ rb, const float* __restrict__ gw,
                                                     int* __restrict__ idx, float* __restrict__ wts,
-                                                    float* __restrict__ gate, int W, int E, int top) {
-  __shared__ float z[MAX_E + 1];
+                                                    float* __restrict__ gate, int W, int E, int top, int scored,
+                                                    const float* __restrict__ corr, int groups, int keep, float wscale) {
+  __shared__ float z[MAX_E + 1], sc[MAX_E], gs[MAX_E];   // logits / choice scores, sigmoid scores, group scores
   const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const T* row = h + static_cast<size_t>(t) * W;
   const int rows = E + (gw != nullptr ? 1 : 0);
@@ -44,7 +48,41 @@ __global__ __launch_bounds__(256) void route_kernel(const T* __restrict__ h, con
     if (lane == 0) z[e] = d + ((e < E && rb) ? rb[e] : 0.f);
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
+  if (threadIdx.x == 0 && scored) {
+    for (int e = 0; e < E; ++e) {
+      sc[e] = 1.0f / (1.0f + expf(-z[e]));
+      z[e] = sc[e] + (corr != nullptr ? corr[e] : 0.f);
+    }
+    if (groups > 1 && keep < groups) {
+      const int per = E / groups;
+      for (int g = 0; g < groups; ++g) {
+        float a = -INFINITY, b = -INFINITY;   // the two largest of the group
+        for (int e = g * per; e < (g + 1) * per; ++e) {
+          const float v = z[e];
+          if (v > a) { b = a; a = v; } else if (v > b) { b = v; }
+        }
+        gs[g] = per > 1 ? a + b : a;
+      }
+      for (int g = 0; g < groups; ++g) {      // a group stays if fewer than `keep` groups come before it
+        int ahead = 0;
+        for (int o = 0; o < groups; ++o) ahead += (gs[o] > gs[g] || (gs[o] == gs[g] && o < g)) ? 1 : 0;
+        if (ahead >= keep)
+          for (int e = g * per; e < (g + 1) * per; ++e) z[e] = -INFINITY;
+      }
+    }
+    float den = 0.f;
+    for (int j = 0; j < top; ++j) {
+      int be = 0;   // (the host checked that `top` experts are allowed)
+      float bv = -INFINITY;
+      for (int e = 0; e < E; ++e)
+        if (z[e] > bv) { bv = z[e]; be = e; }
+      z[be] = -INFINITY;
+      idx[t * top + j] = be;
+      wts[t * top + j] = sc[be];
+      den += sc[be];
+    }
+    for (int j = 0; j < top; ++j) wts[t * top + j] = wts[t * top + j] / (den + 1e-20f) * wscale;
+  } else if (threadIdx.x == 0) {
     if (gw != nullptr) gate[t] = z[E];
     float best0 = 0.f, den = 0.f;
     for (int j = 0; j < top; ++j) {
@@ -412,6 +450,23 @@ __global__ __launch_bounds__(256) void combine_kernel(const T* __restrict__ y, c
 
 BCG_API int bcg_moe_tile_rows() { return TM; }
 
+BCG_API int bcg_moe_route_scored(const void* h, const void* rw, const void* corr, void* idx, void* wts, int T_, int W, int E,
+                                 int top, int groups, int keep, float wscale, int is_f32, void* stream) {
+  if (T_ <= 0) return 0;
+  if (E < 1 || E > MAX_E || top < 1 || top > E || groups < 1 || E % groups || keep < 1 || keep > groups ||
+      top > keep * (E / groups)) return -2;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (is_f32)
+    route_kernel<float><<<T_, 256, 0, s>>>(static_cast<const float*>(h), static_cast<const float*>(rw), nullptr, nullptr,
+                                          static_cast<int*>(idx), static_cast<float*>(wts), nullptr, W, E, top, 1,
+                                          static_cast<const float*>(corr), groups, keep, wscale);
+  else
+    route_kernel<bf16_t><<<T_, 256, 0, s>>>(static_cast<const bf16_t*>(h), static_cast<const float*>(rw), nullptr, nullptr,
+                                           static_cast<int*>(idx), static_cast<float*>(wts), nullptr, W, E, top, 1,
+                                           static_cast<const float*>(corr), groups, keep, wscale);
+  return BCG_CHECK_LAUNCH();
+}
+
 BCG_API int bcg_moe_route(const void* h, const void* rw, const void* rb, const void* gw, void* idx, void* wts, void* gate,
                           int T_, int W, int E, int top, int is_f32, void* stream) {
   if (T_ <= 0) return 0;
@@ -420,11 +475,11 @@ BCG_API int bcg_moe_route(const void* h, const void* rw, const void* rb, const v
   if (is_f32)
     route_kernel<float><<<T_, 256, 0, s>>>(static_cast<const float*>(h), static_cast<const float*>(rw), static_cast<const float*>(rb),
                                          static_cast<const float*>(gw), static_cast<int*>(idx), static_cast<float*>(wts),
-                                         static_cast<float*>(gate), W, E, top);
+                                         static_cast<float*>(gate), W, E, top, 0, nullptr, 1, 1, 1.0f);
   else
     route_kernel<bf16_t><<<T_, 256, 0, s>>>(static_cast<const bf16_t*>(h), static_cast<const float*>(rw), static_cast<const float*>(rb),
                                           static_cast<const float*>(gw), static_cast<int*>(idx), static_cast<float*>(wts),
-                                          static_cast<float*>(gate), W, E, top);
+                                          static_cast<float*>(gate), W, E, top, 0, nullptr, 1, 1, 1.0f);
   return BCG_CHECK_LAUNCH();
 }
 

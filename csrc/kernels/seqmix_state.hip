@@ -431,7 +431,10 @@ __global__ __launch_bounds__(NT) void delta_prepare_kernel(const T* __restrict__
 // columns; the next chunk's loads fly under this chunk's arithmetic.
 struct ScanArgs {
   const float* q; const float* k; const float* g;   // [T, Gq, dim], [T, Gq, dim], [T, H, gd]
-  const void* v; int64_t v_stride;                  // [T, >= H vdim]
+  const void* v; int64_t v_stride;                  // [T, >= H v_head]; head h's values start at h v_head
+  int v_head;                                       // = vdim, or vdim - 1 with unit_last
+  int unit_last;                                    // the state's last column reads a value of 1 for every token (it
+                                                    // accumulates the written keys alone: a normaliser beside the memory)
   const float* beta;                                // [T, H]
   const int* positions; const int* q_start; const int* state_rows;
   float* state;                                     // [n_rows, H, dim, vdim]
@@ -473,7 +476,8 @@ __global__ __launch_bounds__(64 * SCAN_WAVES) void state_scan_kernel(ScanArgs a)
   float S[RPL];
 #pragma unroll
   for (int i = 0; i < RPL; ++i) S[i] = (load_state && rg * RPL + i < dim) ? Sp[static_cast<size_t>(i) * vdim] : 0.f;
-  const T* vbase = static_cast<const T*>(a.v) + h * vdim + (col_ok ? j : 0);
+  const bool unit_col = a.unit_last && j == vdim - 1;
+  const T* vbase = static_cast<const T*>(a.v) + h * a.v_head + ((col_ok && !unit_col) ? j : 0);
 
   // element e of a token is (which of q, k, g; row); rows past dim are zero.  A thread's sources
   // are walked token by token (chunks are loaded in order): one pointer step per element and
@@ -504,7 +508,7 @@ __global__ __launch_bounds__(64 * SCAN_WAVES) void state_scan_kernel(ScanArgs a)
         c.r[tt][n] = (live && src_ok[n]) ? *src[n] : 0.f;
         src[n] += step[n];
       }
-      c.v[tt] = (live && col_ok) ? Elem<T>::ld(*vsrc) : 0.f;
+      c.v[tt] = (live && col_ok) ? (unit_col ? 1.0f : Elem<T>::ld(*vsrc)) : 0.f;
       vsrc += a.v_stride;
       c.be[tt] = 1.0f;
       if (scaled) {
@@ -590,24 +594,28 @@ __global__ __launch_bounds__(64 * SCAN_WAVES) void state_scan_kernel(ScanArgs a)
   }
 }
 
-// o fp32 [T, H, vdim] -> out [T, H vdim]: every head over its root mean square, times w [vdim],
-// times sigmoid(gate[t, h vdim + e]) (gate_kind 0) or silu of it (1) (gate null: none).  One wave per (token, head).
+// o fp32 [T, H, vdim] -> out [T, H vdim]: every head over its root mean square, times w [vdim]
+// (w_head = 0) or w [H vdim] (w_head = vdim), times sigmoid(gate[t, h vdim + e]) (gate_kind 0) or silu
+// of it (1) (gate null: none).  With `floor_` [T, H] a head of o has vdim + 1 columns and is first
+// divided by max(|last column|, floor) + 1e-6 (a memory read beside its normaliser).  One wave per
+// (token, head).
 template <typename T>
 __global__ __launch_bounds__(NT) void head_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ w, float eps,
                                                             const T* __restrict__ gate, int64_t gate_stride,
                                                             T* __restrict__ out, int64_t n_heads_total, int H, int vdim,
-                                                            int gate_kind) {
+                                                            int gate_kind, const float* __restrict__ floor_, int w_head) {
   const int lane = threadIdx.x & 63;
   const int64_t th = static_cast<int64_t>(blockIdx.x) * (NT / 64) + (threadIdx.x >> 6);
   if (th >= n_heads_total) return;
-  const float* x = o + th * vdim;
+  const float* x = o + th * (vdim + (floor_ != nullptr ? 1 : 0));
+  const float pre = floor_ != nullptr ? 1.0f / (fmaxf(fabsf(x[vdim]), floor_[th]) + 1e-6f) : 1.0f;
   float s = 0.f;
-  for (int e = lane; e < vdim; e += 64) s += x[e] * x[e];
-  const float r = 1.0f / sqrtf(wave_sum(s) / vdim + eps);
+  for (int e = lane; e < vdim; e += 64) s += (x[e] * pre) * (x[e] * pre);
+  const float r = pre / sqrtf(wave_sum(s) / vdim + eps);
   const int64_t t = th / H;
   const int h = static_cast<int>(th - t * H);
   for (int e = lane; e < vdim; e += 64) {
-    float v = x[e] * r * w[e];
+    float v = x[e] * r * w[h * w_head + e];
     if (gate != nullptr) {
       const float z = Elem<T>::ld(gate[t * gate_stride + static_cast<int64_t>(h) * vdim + e]);
       v *= gate_kind == 0 ? sigmoidf_(z) : z * sigmoidf_(z);
@@ -768,12 +776,13 @@ BCG_API int bcg_delta_prepare(const void* c, int64_t c_stride, const void* y, in
 BCG_API int bcg_gated_state_scan(const void* q32, const void* k32, const void* g32, const void* v, int64_t v_stride,
                                  const void* beta, const void* positions, const void* q_start, const void* state_rows,
                                  void* state, int n_rows, void* out, int B, int H, int Gq, int dim, int vdim, int gd, int delta,
-                                 int is_f32, void* stream) {
+                                 int unit_last, int is_f32, void* stream) {
   if (B <= 0) return 0;
   if (dim < 1 || dim > 256 || H <= 0 || Gq <= 0 || H % Gq || H > 65535 || (delta && beta == nullptr) || (gd != 1 && gd != dim)) return -2;
+  if (unit_last && (delta || vdim < 2)) return -2;
   ScanArgs a;
   a.q = static_cast<const float*>(q32); a.k = static_cast<const float*>(k32); a.g = static_cast<const float*>(g32);
-  a.v = v; a.v_stride = v_stride; a.beta = static_cast<const float*>(beta);
+  a.v = v; a.v_stride = v_stride; a.v_head = unit_last ? vdim - 1 : vdim; a.unit_last = unit_last; a.beta = static_cast<const float*>(beta);
   a.positions = static_cast<const int*>(positions); a.q_start = static_cast<const int*>(q_start);
   a.state_rows = static_cast<const int*>(state_rows);
   a.state = static_cast<float*>(state); a.out = static_cast<float*>(out);
@@ -784,15 +793,18 @@ BCG_API int bcg_gated_state_scan(const void* q32, const void* k32, const void* g
 }
 
 BCG_API int bcg_head_norm_gate(const void* o32, const void* w, float eps, const void* gate, int64_t gate_stride, void* out,
-                               int T_, int H, int vdim, int gate_kind, int is_f32, void* stream) {
+                               int T_, int H, int vdim, int gate_kind, const void* floor_, int w_head, int is_f32,
+                               void* stream) {
   if (T_ <= 0 || H <= 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int64_t n = static_cast<int64_t>(T_) * H;
   const int grid = static_cast<int>((n + NT / 64 - 1) / (NT / 64));
   const float *o = static_cast<const float*>(o32), *wf = static_cast<const float*>(w);
   BCG_BY_TYPE((head_norm_gate_kernel<float><<<grid, NT, 0, s>>>(o, wf, eps, static_cast<const float*>(gate), gate_stride,
-                                                               static_cast<float*>(out), n, H, vdim, gate_kind)),
+                                                               static_cast<float*>(out), n, H, vdim, gate_kind,
+                                                               static_cast<const float*>(floor_), w_head)),
               (head_norm_gate_kernel<bf16_t><<<grid, NT, 0, s>>>(o, wf, eps, static_cast<const bf16_t*>(gate), gate_stride,
-                                                                static_cast<bf16_t*>(out), n, H, vdim, gate_kind)));
+                                                                static_cast<bf16_t*>(out), n, H, vdim, gate_kind,
+                                                                static_cast<const float*>(floor_), w_head)));
   return BCG_CHECK_LAUNCH();
 }
