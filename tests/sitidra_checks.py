@@ -1,0 +1,320 @@
+"""Checks of the Sitidra mechanisms and engine schedules against the float64 oracle, written once
+for both backends: ``Env("torch", "cpu", ...)`` runs the PyTorch reference ops, ``Env("hip", "cuda",
+...)`` the HIP kernels.  Every mixer is driven alone, over shuffled pages and state rows, whole and
+in portions, with an input of the test's making."""
+import numpy as np
+import torch
+
+import sitidra_cases as C
+import sitidra_oracle as O
+from byzantine_consensus_llm_agents_amd.models.config import SitidraConfig
+from byzantine_consensus_llm_agents_amd.models.sitidra import SitidraModel
+from byzantine_consensus_llm_agents_amd.ops import get_ops
+
+
+class Env:
+    def __init__(self, backend, device, dtype=torch.float32):
+        self.backend, self.device, self.dtype = backend, device, dtype
+        self.ops = get_ops(backend)
+        self.noise = 0.0   # bf16: the worst row error that rounding alone causes in this case (`measure_noise`)
+
+    def measure_noise(self, path, cfg, sd, n=150):
+        """Run the reference ops in this dtype over one prompt: what rounding alone does to the
+        worst row of this configuration."""
+        if self.dtype == torch.float32:
+            return
+        toks = C.tokens(n, cfg["vocab"], 77)
+        ref = C.engine(path, backend="torch", dtype=self.dtype, pool_tokens=max(256, n + 16))
+        got = ref.stream_step([("n", toks, list(range(n)))], end=["n"]).double().numpy()
+        ref.shutdown()
+        want = O.forward(sd, cfg, toks)
+        self.noise = float((np.sqrt(((got - want) ** 2).mean(-1)) / max(float(want.std()), 1e-6)).max())
+
+    def close(self, got, want, tol=None, noise=0.0):
+        """fp32: elementwise.  bf16: the row error relative to the spread of the expected values."""
+        got, want = got.detach().double().cpu().numpy(), np.asarray(want)
+        assert got.shape == want.shape, (got.shape, want.shape)
+        noise = max(noise, self.noise)
+        if self.dtype == torch.float32:
+            tol = tol or 2e-3
+            np.testing.assert_allclose(got, want, atol=tol, rtol=tol)
+        else:
+            err = np.sqrt(((got - want) ** 2).mean(-1)) / max(float(want.std()), 1e-6)
+            assert float(err.max()) < max(0.15, 1.5 * noise), float(err.max())
+            assert float(np.quantile(err, 0.9)) < max(0.08, noise), float(np.quantile(err, 0.9))
+            assert float(np.median(err)) < 0.04, float(np.median(err))
+
+    def t(self, x, dtype=None):
+        return torch.as_tensor(np.asarray(x)).to(device=self.device, dtype=dtype or self.dtype, copy=True)
+
+
+def rand_bf16(g, *shape, scale=1.0):
+    return (torch.randn(*shape, generator=g) * scale).to(torch.bfloat16).float()
+
+
+# ------------------------------------------------------------------ streams and layer norms
+def check_streams(env, S, W=44, T=7):
+    g = torch.Generator().manual_seed(S)
+    f = lambda a: env.t(a, torch.float32)  # noqa: E731
+    table = rand_bf16(g, 11, W, scale=2.0)
+    r1, r2, o1 = rand_bf16(g, S), rand_bf16(g, S), rand_bf16(g, S)
+    mix = rand_bf16(g, S, S)
+    w1, w2 = rand_bf16(g, W), rand_bf16(g, W)
+    toks = [3, 0, 10, 3, 7, 1, 2][:T]
+    X, h = env.ops.hyper_embed_norm(torch.tensor(toks, dtype=torch.int32, device=env.device), env.t(table), S, f(r1), f(w1), 1e-5,
+                                    env.dtype)
+    x0 = table.double().numpy()[toks]
+    xs = np.stack([x0] * S)
+    env.close(X, xs.transpose(1, 0, 2), 1e-6)
+    env.close(h, O.layer_norm(np.tensordot(r1.double().numpy(), xs, 1), w1.double().numpy(), 1e-5), 1e-5)
+    # a sublayer output in two parts (activation-typed and fp32), the next read and its norm
+    ya, yb = rand_bf16(g, T, W), rand_bf16(g, T, W)
+    sd = {"in": r1.double().numpy(), "mix": mix.double().numpy(), "out": o1.double().numpy()}
+    want = O.hyper_sublayer(sd, "", xs, lambda u: ya.double().numpy() + yb.double().numpy())
+    h2 = env.ops.hyper_update_norm(X, [env.t(ya), f(yb)], f(mix), f(o1), f(r2), f(w2), 1e-5, env.dtype)
+    env.close(X, want.transpose(1, 0, 2), 1e-5)
+    env.close(h2, O.layer_norm(np.tensordot(r2.double().numpy(), want, 1), w2.double().numpy(), 1e-5), 2e-5)
+    # no read asked for: only the streams change
+    want2 = O.hyper_sublayer(sd, "", want, lambda u: ya.double().numpy())
+    assert env.ops.hyper_update_norm(X, [env.t(ya)], f(mix), f(o1), None, None, 1e-5, env.dtype) is None
+    env.close(X, want2.transpose(1, 0, 2), 1e-4)
+
+
+# ------------------------------------------------------------------ one mixer alone
+def _model(env, layers, width, seed, streams=2):
+    cfg = SitidraConfig.from_dict(C.config(layers, width=width, vocab=29, streams=streams), "t")
+    model = SitidraModel(cfg, env.ops, env.device, env.dtype)
+    return cfg, model, model.random_state_dict(seed, std=0.2)
+
+
+def run_mixer(env, layers, T, cuts=None, craft=None, seed=0, width=40):
+    """Drive the LAST layer's mixer alone over the portions ``cuts`` of one sequence (an earlier
+    attention layer that lends its values runs too, from an input of its own).  ``craft(sd, hs)`` may
+    edit the weights and the per-layer inputs.  Returns (got [T, W], want [T, W])."""
+    cfg, model, sd = _model(env, layers, width, seed)
+    g = torch.Generator().manual_seed(seed + 100)
+    hs = [rand_bf16(g, T, width) for _ in layers]
+    if craft:
+        craft(sd, hs)
+    model.load_hf_state_dict(sd)
+    sd64 = O.to_f64(sd)
+    eps = cfg.rms_eps
+    last = len(layers) - 1
+    spec = layers[last]
+    p = f"l{last}.mix."
+    h64 = hs[last].double().numpy()
+    if spec["type"] == "attention":
+        v_first = None
+        if spec["mixer"].get("v_mix") and model.v_lender != last:
+            j = model.v_lender
+            v_first = O.attention_values(sd64, f"l{j}.mix.", layers[j]["mixer"], hs[j].double().numpy())
+        want = O.attention(sd64, p, spec["mixer"], h64, eps, v_first)
+    else:
+        want = O.mlstm(sd64, p, spec["mixer"], h64, eps)
+    pages = C.Pages([T, 5, T], seed=seed, device=env.device)   # sequence 2 is ours: state row 2
+    ks, vs = model.alloc_kv(pages.num_blocks, 16, env.dtype)
+    state = model.alloc_state(4)
+    for L in state["layers"]:
+        if L is not None:   # stale state of an earlier owner
+            L["S"].fill_(3.0)
+            L["m"].fill_(-7.0)
+    at, outs = 0, []
+    for c in cuts or [T]:
+        meta = pages.meta([(2, at, c)])
+        meta.state = state
+        lent = []
+        for i, l in enumerate(layers):
+            m, L = model.cfg.layers[i].mixer, model.layers[i]
+            h = env.t(hs[i][at:at + c])
+            if l["type"] == "attention" and (i == last or i == model.v_lender):
+                y = model._attention(i, m, L, h, meta, ks[i], vs[i], None, lent)
+            elif i == last:
+                y = model._mlstm(m, L, state["layers"][i], h, meta, None)
+            if i == last:
+                outs.append(y)
+        at += c
+    return torch.cat(outs), want
+
+
+def loud_value(pos, factor=100.0):
+    """Input row ``pos`` scaled up.  Keys are unit vectors whatever the input's size, values are
+    not: the row's value is ``factor`` times the others, so a query that sees this key has an
+    output dominated by it, and dropping or adding the key shows."""
+    def craft(sd, hs):
+        for h in hs:
+            h[pos] *= factor
+    return craft
+
+
+def check_chunk_edge(env, chunk=9, T=40, cuts=None, seed=5):
+    """The loud row is the FIRST of a chunk: every position of that chunk sees it, the last position
+    of the chunk before and the first of the chunk after do not."""
+    loud = 2 * chunk
+    m = C.attn(2, 1, 16, 16, chunk, 8, scale=0.05)   # a flat softmax: every visible key carries weight
+    got, want = run_mixer(env, [C.layer("attention", m, 0)], T, cuts, loud_value(loud), seed=seed)
+    env.close(got, want)
+    inside, outside = want[loud + chunk - 1], want[loud + chunk]
+    assert np.abs(inside).max() > 4 * np.abs(outside).max()   # the edge is visible far above the tolerance
+    assert np.abs(want[loud]).max() > 4 * np.abs(want[loud - 1]).max()
+    return got
+
+
+def check_router(env, E, top, groups, keep, scale, W=40, T=64, corr_shift=0.0):
+    g = torch.Generator().manual_seed(E * 100 + top * 10 + groups)
+    sd = {"router": rand_bf16(g, E, W, scale=0.4), "correction": rand_bf16(g, E, scale=0.3) + corr_shift}
+    h = rand_bf16(g, T, W)
+    f = {"router": {"experts": E, "top": top, "scale": scale}}
+    if groups:
+        f["router"]["groups"] = {"count": groups, "keep": keep}
+    want = O.route(O.to_f64(sd), "", f, h.double().numpy())
+    idx, wts = env.ops.moe_route_scored(env.t(h), env.t(sd["router"], torch.float32), env.t(sd["correction"], torch.float32), top,
+                                        groups or 1, keep if groups else 1, scale)
+    assert idx.shape == (T, top) and idx.dtype == torch.int32
+    n_diff = 0
+    for t, (ids, w) in enumerate(want):
+        got_ids = idx[t].cpu().tolist()
+        if sorted(got_ids) != sorted(ids):   # bf16 inputs are exact here, so only a true tie could differ
+            n_diff += 1
+            continue
+        order = [got_ids.index(e) for e in ids]
+        np.testing.assert_allclose(wts[t].double().cpu().numpy()[order], w, rtol=1e-4, atol=1e-6)
+    assert n_diff == 0, n_diff
+
+
+def check_experts(env, E, top, groups, keep, ff, shared, W=40, T=23, scale=1.7):
+    """Routing, routed gated experts and the always-on expert against the oracle's feed-forward."""
+    spec = C.layer("mlstm", C.mlstm(1, 4, 4), ff, E, top, (groups, keep) if groups else None, scale, shared)
+    cfg, model, sd = _model(env, [spec], W, seed=E + top)
+    model.load_hf_state_dict(sd)
+    g = torch.Generator().manual_seed(E)
+    h = rand_bf16(g, T, W)
+    want = O.feed_forward(O.to_f64(sd), "l0.mlp.", spec["mlp"], h.double().numpy())
+    parts = model._experts(cfg.layers[0].mlp, model.layers[0], env.t(h))
+    got = parts[0].float()
+    for p in parts[1:]:
+        got = got + p.float()
+    env.close(got, want)
+
+
+# ------------------------------------------------------------------ engine schedules
+def whole_prompt(env, cfg, sd, eng, n=45):
+    toks = C.tokens(n, cfg["vocab"], 1)
+    env.close(eng.stream_step([("a", toks, list(range(n)))], end=["a"]), O.forward(sd, cfg, toks))
+
+
+def stream_after_every_layer(env, cfg, sd, eng):
+    toks = C.tokens(19, cfg["vocab"], 2)
+    want = []
+    O.forward(sd, cfg, toks, want)
+    pages = C.Pages([19], device=env.device)
+    meta = pages.meta([(0, 0, 19)])
+    meta.state = eng.model.alloc_state(2)
+    k, v = eng.model.alloc_kv(pages.num_blocks, 16, env.dtype)
+    got = []
+    eng.model.forward(torch.tensor(toks, dtype=torch.int32, device=env.device), meta, k, v, trace=got)
+    assert len(got) == len(want) == len(cfg["layers"])
+    for a, b in zip(got, want):
+        env.close(a, b)
+
+
+def prefill_then_token_by_token(env, cfg, sd, eng, n=70, first=30):
+    toks = C.tokens(n, cfg["vocab"], 3)
+    want = O.forward(sd, cfg, toks)
+    env.close(eng.stream_step([("d", toks[:first], [0, 1, first - 1])]), want[[0, 1, first - 1]])
+    got = [eng.stream_step([("d", toks[p:p + 1], [0])], end=["d"] if p == n - 1 else []) for p in range(first, n)]
+    env.close(torch.cat(got), want[first:])   # crosses page borders and every chunk's edge
+
+
+def first_tokens_one_by_one(env, cfg, sd, eng):
+    toks = C.tokens(7, cfg["vocab"], 4)
+    want = O.forward(sd, cfg, toks)
+    got = [eng.stream_step([("f", toks[p:p + 1], [0])], end=["f"] if p == 6 else []) for p in range(7)]
+    env.close(torch.cat(got), want)
+
+
+def portions(env, cfg, sd, eng, sizes):
+    n = sum(sizes)
+    toks = C.tokens(n, cfg["vocab"], 5)
+    want = O.forward(sd, cfg, toks)
+    at, got = 0, []
+    for i, s in enumerate(sizes):
+        got.append(eng.stream_step([("p", toks[at:at + s], list(range(s)))], end=["p"] if i == len(sizes) - 1 else []))
+        at += s
+    env.close(torch.cat(got), want)
+
+
+def mixed_batches_and_reuse(env, cfg, sd, eng, lens=(70, 33, 18, 64, 41, 90, 5, 36)):
+    """Up to four live requests, portions beside single tokens, rows sitting out; twice as many
+    requests as state rows over a pool smaller than the work: pages and rows are used again."""
+    reqs = {f"r{i}": C.tokens(n, cfg["vocab"], 10 + i) for i, n in enumerate(lens)}
+    want = {k: O.forward(sd, cfg, t) for k, t in reqs.items()}
+    at = {k: 0 for k in reqs}
+    waiting, live, step = list(reqs), [], 0
+    free_at_start = eng.blocks.num_free_blocks
+    got, expect = [], []
+    while waiting or live:
+        while waiting and len(live) < 4:
+            live.append(waiting.pop(0))
+        entries, end = [], []
+        for j, k in enumerate(live):
+            if (step + j) % 5 == 4 and at[k] > 0:
+                continue
+            take = [1, 2, 16, 7, 1, 19][(step + j) % 6] if at[k] > 0 else [20, 3, 16][j % 3]
+            take = min(take, len(reqs[k]) - at[k])
+            entries.append((k, reqs[k][at[k]:at[k] + take], list(range(take))))
+            expect.append(want[k][at[k]:at[k] + take])
+            at[k] += take
+            if at[k] == len(reqs[k]):
+                end.append(k)
+        if entries:
+            got.append(eng.stream_step(entries, end))
+        live = [k for k in live if k not in end]
+        step += 1
+    env.close(torch.cat(got), np.concatenate(expect))
+    assert eng.blocks.num_free_blocks == free_at_start and not any(eng.slots)
+    assert sum(lens) > 16 * free_at_start / 2
+
+
+def greedy_generation(env, cfg, sd, eng, tie=1e-3):
+    prompts = [C.tokens(n, cfg["vocab"], 20 + n) for n in (9, 31, 16, 2, 40, 23)]
+    budgets = (6, 4, 17, 5, 3, 11)
+    outs = eng.generate_ids(prompts, max_tokens=list(budgets), temperature=0.0)
+    for p, out, n in zip(prompts, outs, budgets):
+        assert len(out) == n
+        seq = list(p)
+        for tok in out:
+            logits = O.forward(sd, cfg, seq)[-1]
+            top2 = np.sort(logits)[-2:]
+            if float(top2[1] - top2[0]) < tie * max(1.0, float(logits.std())):
+                break  # a near tie: either token is a correct greedy step
+            assert tok == int(logits.argmax())
+            seq.append(tok)
+
+
+def drawn_configuration(env, tmp_path, seed, pool_tokens=256):
+    cfg = C.random_config(seed)
+    path = str(tmp_path / "m")
+    sd = O.to_f64(C.checkpoint(cfg, path, seed=seed))
+    a, b = C.tokens(60, cfg["vocab"], seed), C.tokens(23, cfg["vocab"], seed + 100)
+    wa, wb = O.forward(sd, cfg, a), O.forward(sd, cfg, b)
+    noise = 0.0
+    if env.dtype != torch.float32:   # what bf16 rounding alone does to this configuration's worst row
+        ref = C.engine(path, backend="torch", dtype=env.dtype, pool_tokens=pool_tokens)
+        r = ref.stream_step([("w", a, list(range(60)))], end=["w"]).double().numpy()
+        ref.shutdown()
+        noise = float((np.sqrt(((r - wa) ** 2).mean(-1)) / max(float(wa.std()), 1e-6)).max())
+    eng = C.engine(path, backend=env.backend, dtype=env.dtype, pool_tokens=pool_tokens)
+    try:
+        env.close(eng.stream_step([("w", a, list(range(60)))], end=["w"]), wa, noise=noise)
+        at, got, want = 0, [], []
+        for i, s in enumerate([3, 2, 30, 1, 1, 17, 2, 4]):
+            entries = [("a", a[at:at + s], list(range(s))), ("b", b[i:i + 1], [0])]
+            want += [wa[at:at + s], wb[i:i + 1]]
+            at += s
+            got.append(eng.stream_step(entries))
+        env.close(torch.cat(got), np.concatenate(want), noise=noise)
+        assert at == 60
+        eng.stream_step([("b", b[8:], [])], end=["a", "b"])
+        assert not any(eng.slots)
+    finally:
+        eng.shutdown()
