@@ -121,8 +121,11 @@ def parse(argv=None):
                     help="rehearsal on a 1-GPU box: every rank on cuda:0, gloo process group, the xGMI "
                          "all-reduce kernels forced over IPC peer buffers (never for measurements)")
     ap.add_argument("--verbose", action="store_true")
+    ap.add_argument("--families", default="",
+                    help="with --family-compare: only these families and their kernel groups (comma-separated, of mofidra, "
+                         "padadra, mabivik, sitidra, decoder; default: all)")
     ap.add_argument("--family-compare", action="store_true",
-                    help="instead of the headline workload: prefill / decode tokens/s of the Mofidra, Padadra and Mabivik families beside "
+                    help="instead of the headline workload: prefill / decode tokens/s of the Mofidra, Padadra, Mabivik and Sitidra families beside "
                          "the Qwen3-style decoder at equal layer sizes, and their hot kernels against the roofline "
                          "(one GPU, random weights; utils/family_bench.py)")
     return ap.parse_args(argv)
@@ -388,7 +391,7 @@ def main(argv=None):
     args = parse(argv)
     if args.family_compare:
         from byzantine_consensus_llm_agents_amd.utils.family_bench import run
-        print(json.dumps(run()), flush=True)
+        print(json.dumps(run(families=[f for f in args.families.split(",") if f] or None)), flush=True)
         return 0
     world = int(os.environ.get("WORLD_SIZE", "0") or 0)
     if world == 0 and args.gpus > 1:

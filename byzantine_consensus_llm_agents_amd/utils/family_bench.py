@@ -1,4 +1,4 @@
-"""Prefill / decode throughput of the Mofidra, Padadra and Mabivik families beside the Qwen3-style decoder
+"""Prefill / decode throughput of the Mofidra, Padadra, Mabivik and Sitidra families beside the Qwen3-style decoder
 at equal layer sizes (random weights, synthetic tokens), and the hot kernels against their
 rooflines.  ``bench.py --family-compare`` prints the result as one JSON line.
 
@@ -24,6 +24,14 @@ head; 4-tap convolutions; every feed-forward routes top-2 of 8 gated experts of 
 (Mofidra's MoE variant is its relative there); a 256-wide token input per layer.  Its closest
 relative is Padadra (fp32 stream, windowed attention beside recurrences, the same state tables).
 
+Sitidra at equal size: the same width and query / KV head counts; four layers (attention, matrix
+memory, attention, matrix memory) over four hyper-connection streams; the attention has 128 query /
+key and 128 value features per head, rotary on 64 of them, unit-norm heads, 512-position chunks and
+mixed values; the matrix memory has the query-head count of 128 x 128 memories (129 state columns
+with the normaliser); every feed-forward routes top-2 of 8 gated experts of ff/4 by sigmoid score
+inside 2 of 4 groups, plus a shared expert of ff/2.  Its closest relative is Mabivik (fp32
+stream, masked attention beside recurrences on the same scan kernel, the same gated experts).
+
 Rooflines: 2.5 PFLOP/s dense bf16 MFMA, 8 TB/s HBM.  A kernel's ``roof_frac`` is
 max(flops / peak, bytes / bandwidth) / measured time.  The recurrence runs on the vector ALUs:
 its compute roof is 157 TFLOP/s fp32.
@@ -34,10 +42,11 @@ import time
 
 import torch
 
-from ..models.config import MabivikConfig, MofidraConfig, ModelConfig, PadadraConfig
+from ..models.config import MabivikConfig, MofidraConfig, ModelConfig, PadadraConfig, SitidraConfig
 from ..models.mabivik import MabivikModel
 from ..models.mofidra import MofidraModel
 from ..models.padadra import PadadraModel
+from ..models.sitidra import SitidraModel
 from ..models.transformer import AttnMeta, DecoderModel
 from ..ops import get_ops
 
@@ -93,6 +102,19 @@ def mabivik_config(s) -> MabivikConfig:
     return MabivikConfig.from_dict({"architecture": "Mabivik", "width": W, "vocab": s["vocab"], "embedding": {"scale": 1.0},
                                     "norm": {"eps": 1e-5}, "logit_scale": 1.0, "token_side": {"dim": 256}, "layers": layers},
                                    "mabivik-bench")
+
+
+def sitidra_config(s) -> SitidraConfig:
+    H, G, W = s["heads"], s["kv_heads"], s["width"]
+    att = {"heads": H, "kv_heads": G, "dim": 128, "vdim": 128, "scale": 0.088, "rot": {"dims": 64, "base": 1e6},
+           "mask": {"size": 512}, "v_mix": True}
+    mem = {"heads": H, "dim": 128, "vdim": 128, "gate_cap": 15.0}
+    mlp = {"kind": "moe", "expert": {"ff": s["ff"] // 4},
+           "router": {"experts": 8, "top": 2, "scale": 2.0, "groups": {"count": 4, "keep": 2}}, "shared": {"ff": s["ff"] // 2}}
+    layers = [{"type": "attention" if i % 2 == 0 else "mlstm", "mixer": att if i % 2 == 0 else mem, "mlp": mlp}
+              for i in range(s["layers"])]
+    return SitidraConfig.from_dict({"architecture": "Sitidra", "width": W, "vocab": s["vocab"], "norm": {"eps": 1e-5},
+                                    "streams": 4, "logit_softcap": 50.0, "layers": layers}, "sitidra-bench")
 
 
 def decoder_config(s) -> ModelConfig:
@@ -474,7 +496,125 @@ def latent_kernels(s, dev):
     return out
 
 
-def run(sizes=("w2048", "w4096"), kernels=True) -> dict:
+def hyper_kernels(s, dev):
+    """Sitidra's kernels beside the like kernels of Mabivik, Padadra and Mofidra at the same shapes."""
+    ops = get_ops("hip")
+    H, G, W = s["heads"], s["kv_heads"], s["width"]
+    bf = torch.bfloat16
+    out = {}
+    n, ctx, chunk = 8, 1024, 512
+    T, b = n * ctx, 64
+    meta, nb = step_meta(n, ctx, ctx, 64, dev, True)
+    dmeta, nbd = step_meta(b, ctx, 1, 64, dev, True)
+    nb = max(nb, nbd)
+    pairs = sum(i % chunk + 1 for i in range(ctx)) * n      # (query, key) pairs under the chunk mask
+    pairs_w = sum(min(i + 1, chunk) for i in range(ctx)) * n  # ... under a window of the same size
+    # ---- prefill attention, 8 x 1024: 512-position chunks against a 512-key window (one kernel, two masks) ----
+    q = torch.randn(T, H, 128, device=dev, dtype=bf)
+    kc, vc = torch.randn(nb, G, BS, 128, device=dev, dtype=bf), torch.randn(nb, G, 128, BS, device=dev, dtype=bf)
+    io = T * H * 256 * 2 + T * G * 256 * 2
+    t = _time(lambda: ops.multimap_attention(q, kc, vc, meta, 0.088, 1, 0.0, -1.0, 1.0, 128, 0, None, chunk))
+    out["prefill_attention"] = {"sitidra_ms": round(t * 1e3, 3), "sitidra_roof_frac": _roof(2 * H * 256 * pairs, io, t)}
+    sink = torch.randn(H, device=dev)
+    t = _time(lambda: ops.multimap_attention(q, kc, vc, meta, 0.088, 1, 0.0, -1.0, 1.0, 128, chunk, sink))
+    out["prefill_attention"].update({"padadra_ms": round(t * 1e3, 3), "padadra_roof_frac": _roof(2 * H * 256 * pairs_w, io, t)})
+    # ---- decode attention, 64 rows at position 1023: the chunk's 512 keys against the window's ----
+    qd = torch.randn(b, H, 128, device=dev, dtype=bf)
+    t = _graph_time(lambda: ops.multimap_attention(qd, kc, vc, dmeta, 0.088, 1, 0.0, -1.0, 1.0, 128, 0, None, chunk), iters=50)
+    out["decode_attention"] = {"sitidra_ms": round(t * 1e3, 4),
+                               "sitidra_roof_frac": _roof(2 * H * 256 * b * chunk, b * chunk * G * 256 * 2, t)}
+    t = _graph_time(lambda: ops.multimap_attention(qd, kc, vc, dmeta, 0.088, 1, 0.0, -1.0, 1.0, 128, chunk, sink), iters=50)
+    out["decode_attention"].update({"padadra_ms": round(t * 1e3, 4),
+                                    "padadra_roof_frac": _roof(2 * H * 256 * b * chunk, b * chunk * G * 256 * 2, t)})
+    # ---- stream update + next read + layer norm, 8192 rows x 4 streams, against the one-stream residual kernels ----
+    S = 4
+    X = torch.randn(T, S, W, device=dev)
+    a, p32 = torch.randn(T, W, device=dev, dtype=bf), torch.randn(T, W, device=dev)
+    mix, ow, rw, nw = torch.randn(S, S, device=dev) * 0.3, torch.randn(S, device=dev), torch.randn(S, device=dev), torch.randn(W, device=dev)
+    t = _time(lambda: ops.hyper_update_norm(X, [a], mix, ow, rw, nw, 1e-5, bf), iters=20)
+    out["residual_norm"] = {"sitidra_ms": round(t * 1e3, 4), "sitidra_roof_frac": _roof(0, T * W * (8 * S + 2 + 2), t)}
+    t = _time(lambda: ops.hyper_update_norm(X, [a, p32], mix, ow, rw, nw, 1e-5, bf), iters=20)
+    out["residual_norm_two_parts"] = {"sitidra_ms": round(t * 1e3, 4), "sitidra_roof_frac": _roof(0, T * W * (8 * S + 2 + 4 + 2), t)}
+    x32 = torch.randn(T, W, device=dev)
+    w1, b1, w2, b2 = (torch.randn(W, device=dev) for _ in range(4))
+    t = _time(lambda: ops.residual_post_norm(x32, a, ("dyt", 0.5, w1, b1), ("dyt", 0.7, w2, b2), bf), iters=20)
+    out["residual_norm"].update({"mabivik_ms": round(t * 1e3, 4), "mabivik_roof_frac": _roof(0, T * W * (4 + 4 + 2 + 2), t)})
+    t = _time(lambda: ops.residual_add_rmsnorm32(x32, [a], w1, 1e-5, 1.0, bf), iters=20)
+    out["residual_norm"].update({"mofidra_ms": round(t * 1e3, 4), "mofidra_roof_frac": _roof(0, T * W * (4 + 4 + 2 + 2), t)})
+    del X, x32, p32
+    # ---- cache write, 8192 rows: rotary + unit-norm heads + mixed values against Padadra's and Mofidra's rotary writes ----
+    width = (H + G) * 128 + G * 128
+    y = torch.randn(T, width + H, device=dev, dtype=bf)
+    vf = torch.randn(T, G * 128, device=dev, dtype=bf)
+    inv = torch.rand(32, device=dev)
+    kz, vz = torch.zeros(nb, G, BS, 128, device=dev, dtype=bf), torch.zeros(nb, G, 128, BS, device=dev, dtype=bf)
+    t = _graph_time(lambda: ops.rope_norm_kv_write(y, meta.positions, meta.slots, H, G, 128, 128, inv, 1e-5, vf, 0.3, kz, vz), iters=50)
+    out["cache_write"] = {"sitidra_ms": round(t * 1e3, 4), "sitidra_roof_frac": _roof(0, T * (width * 2 + G * 128) * 2, t)}
+    qn, kn, vinv = torch.ones(H * 128, device=dev), torch.ones(G * 128, device=dev), torch.rand(64, device=dev)
+    t = _graph_time(lambda: ops.rope_pairs_kv_write(y, meta.positions, meta.slots, H, G, 128, 128, qn, kn, 1e-5, inv, vinv, kz, vz), iters=50)
+    out["cache_write"].update({"padadra_ms": round(t * 1e3, 4), "padadra_roof_frac": _roof(0, T * width * 2 * 2, t)})
+    t = _graph_time(lambda: ops.rope_multi_kv_write(y, meta.positions, meta.slots, H, G, 1, 128, 128, inv, kz, vz), iters=50)
+    out["cache_write"].update({"mofidra_ms": round(t * 1e3, 4), "mofidra_roof_frac": _roof(0, T * width * 2 * 2, t)})
+    # ---- output gate: one gate per head against one per feature ----
+    att, gh, gf = torch.randn(T, H * 128, device=dev, dtype=bf), torch.randn(T, H, device=dev, dtype=bf), torch.randn(T, H * 128, device=dev, dtype=bf)
+    t = _time(lambda: ops.gate_mul(att, gh, "sigmoid", 128), iters=20)
+    out["output_gate"] = {"sitidra_ms": round(t * 1e3, 4), "sitidra_roof_frac": _roof(0, T * H * 128 * 2 * 2, t)}
+    t = _time(lambda: ops.gate_mul(att, gf, "sigmoid"), iters=20)
+    out["output_gate"].update({"mabivik_ms": round(t * 1e3, 4), "mabivik_roof_frac": _roof(0, T * H * 128 * 2 * 3, t)})
+    # ---- the memory: gates + running maximum, the scan with the normaliser column, the output norm ----
+    fused = 2 * H * 128 + 2 * H * 128 + 2 * H
+    Hs = 2 * W // 128
+    for name, rows_, m_ in (("prefill", T, meta), ("decode", b, dmeta)):
+        nseq = m_.q_start.numel() - 1
+        m_.state_rows = torch.arange(nseq, dtype=torch.int32, device=dev)
+        timer = (lambda f: _time(f, iters=10)) if name == "prefill" else (lambda f: _graph_time(f, iters=50))
+        yf = torch.randn(rows_, fused, device=dev, dtype=bf)
+        ib, fb = torch.zeros(H, device=dev), torch.ones(H, device=dev)
+        m_state = torch.zeros(max(n, b) + 1, H, device=dev)
+        off_i = 4 * H * 128
+        t = timer(lambda: ops.exp_gate_prepare(yf, 0, H * 128, off_i, off_i + H, ib, fb, 15.0, 128 ** -0.5, H, 128, m_, m_state))
+        entry = {"sitidra_ms": round(t * 1e3, 4), "sitidra_roof_frac": _roof(0, rows_ * (2 * H * 128 * (2 + 4) + 2 * H * 2 + 3 * H * 4), t)}
+        ys = torch.randn(rows_, 2 * Hs * 128 + 2 * 2 * 128 + Hs, device=dev, dtype=bf)
+        dtb, al = torch.zeros(Hs, device=dev), torch.zeros(Hs, device=dev)
+        t = timer(lambda: ops.ssm_prepare(ys, Hs * 128, ys, 2 * Hs * 128 + 4 * 128, dtb, al, Hs, 2, 128))
+        entry.update({"mabivik_ms": round(t * 1e3, 4), "mabivik_roof_frac": _roof(0, rows_ * (4 * 128 * (2 + 4) + Hs * (2 + 8)), t)})
+        out[f"gate_prepare_{name}"] = entry
+        q32, k32, dec, wr, fl = ops.exp_gate_prepare(yf, 0, H * 128, off_i, off_i + H, ib, fb, 15.0, 128 ** -0.5, H, 128, m_, m_state)
+        v = yf[:, 2 * H * 128:3 * H * 128]
+        Sm = torch.zeros(max(n, b) + 1, H, 128, 129, device=dev)
+        t = timer(lambda: ops.gated_state_scan(q32, k32, dec, v, wr, m_, Sm, False, True))
+        flops = rows_ * H * 128 * 129 * 6
+        io = rows_ * (2 * H * 128 * 4 + H * 8 + H * 128 * 2 + H * 129 * 4) + nseq * H * 128 * 129 * 4 * 2
+        entry = {"sitidra_ms": round(t * 1e3, 4), "sitidra_roof_frac": round(max(flops / PEAK_VALU, io / PEAK_BW) / t, 4)}
+        qs, ks = torch.randn(rows_, 2, 128, device=dev) * 0.1, torch.randn(rows_, 2, 128, device=dev) * 0.1
+        gs, dts = torch.rand(rows_, H, 1, device=dev), torch.rand(rows_, H, device=dev)
+        Ss = torch.zeros(max(n, b) + 1, H, 128, 128, device=dev)
+        t = timer(lambda: ops.gated_state_scan(qs, ks, gs, v, dts, m_, Ss, False))   # the state-space form at the same head count
+        flops = rows_ * H * 128 * 128 * 6
+        io = rows_ * (2 * 2 * 128 * 4 + H * 8 + H * 128 * 2 + H * 128 * 4) + nseq * H * 128 * 128 * 4 * 2
+        entry.update({"mabivik_ms": round(t * 1e3, 4), "mabivik_roof_frac": round(max(flops / PEAK_VALU, io / PEAK_BW) / t, 4)})
+        out[f"memory_scan_{name}"] = entry
+        del Sm, Ss
+    o33 = torch.randn(T, H, 129, device=dev)
+    o32 = torch.randn(T, H, 128, device=dev)
+    fl, z = torch.rand(T, H, device=dev), torch.randn(T, H * 128, device=dev, dtype=bf)
+    wn, wh = torch.randn(H * 128, device=dev), torch.randn(128, device=dev)
+    t = _time(lambda: ops.head_norm_gate(o33, wn, 1e-5, z, bf, "sigmoid", fl), iters=20)
+    out["recurrent_out_norm"] = {"sitidra_ms": round(t * 1e3, 4), "sitidra_roof_frac": _roof(0, T * H * (129 * 4 + 4 + 128 * 4), t)}
+    t = _time(lambda: ops.head_norm_gate(o32, wh, 1e-5, z, bf, "silu"), iters=20)
+    out["recurrent_out_norm"].update({"mabivik_ms": round(t * 1e3, 4), "mabivik_roof_frac": _roof(0, T * H * 128 * (4 + 2 + 2), t)})
+    # ---- router: sigmoid scores with groups against the softmax over the chosen ----
+    E = 8
+    h = torch.randn(T, W, device=dev, dtype=bf)
+    rw_, corr = torch.randn(E, W, device=dev) * 0.05, torch.randn(E, device=dev) * 0.1
+    t = _time(lambda: ops.moe_route_scored(h, rw_, corr, 2, 4, 2, 2.0), iters=20)
+    out["router"] = {"sitidra_ms": round(t * 1e3, 4), "sitidra_roof_frac": _roof(2 * T * E * W, T * W * 2, t)}
+    t = _time(lambda: ops.moe_route(h, rw_, corr, 2), iters=20)
+    out["router"].update({"mofidra_ms": round(t * 1e3, 4), "mofidra_roof_frac": _roof(2 * T * E * W, T * W * 2, t)})
+    return out
+
+
+def run(sizes=("w2048", "w4096"), kernels=True, families=None) -> dict:
     dev = torch.device("cuda", torch.cuda.current_device())
     ops = get_ops("hip")
     ops.prepare_device(dev)
@@ -487,16 +627,20 @@ def run(sizes=("w2048", "w4096"), kernels=True) -> dict:
                                  ("mofidra_moe", lambda: MofidraModel(mofidra_config(s, True), ops, dev)),
                                  ("padadra", lambda: PadadraModel(padadra_config(s), ops, dev)),
                                  ("mabivik", lambda: MabivikModel(mabivik_config(s), ops, dev)),
+                                 ("sitidra", lambda: SitidraModel(sitidra_config(s), ops, dev)),
                                  ("decoder", lambda: DecoderModel(decoder_config(s), ops, dev))):
+                if families and label.split("_")[0] not in families:
+                    continue
                 model = build()
                 model.init_random(seed=1, std=0.02)
                 entry[label] = model_throughput(model)
                 del model
                 torch.cuda.empty_cache()
-            if kernels:
-                entry["kernels"] = kernel_pairs(s, dev)
-                entry["state_kernels"] = state_kernels(s, dev)
-                entry["latent_kernels"] = latent_kernels(s, dev)
+            groups = (("mofidra", "kernels", kernel_pairs), ("padadra", "state_kernels", state_kernels),
+                      ("mabivik", "latent_kernels", latent_kernels), ("sitidra", "hyper_kernels", hyper_kernels))
+            for family, key, fn in groups if kernels else ():
+                if not families or family in families:
+                    entry[key] = fn(s, dev)
             result["sizes"][name] = entry
     return result
 

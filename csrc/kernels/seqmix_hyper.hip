@@ -38,18 +38,58 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
 __device__ __forceinline__ float sigmoidf_(float z) { return 1.0f / (1.0f + expf(-z)); }
 __device__ __forceinline__ float log_sigmoidf_(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
+// V consecutive elements (V = 4: one 16-byte or 8-byte access, the caller checked the alignment).
+template <typename T, int V> struct Pack;
+template <typename T> struct Pack<T, 1> {
+  typedef float vec;
+  static __device__ __forceinline__ float ld(const T* p) { return Elem<T>::ld(*p); }
+  static __device__ __forceinline__ void st(T* p, float v) { *p = Elem<T>::st(v); }
+  static __device__ __forceinline__ float get(float v, int) { return v; }
+  static __device__ __forceinline__ void set(float& v, int, float x) { v = x; }
+};
+template <> struct Pack<float, 4> {
+  typedef f32x4 vec;
+  static __device__ __forceinline__ f32x4 ld(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
+  static __device__ __forceinline__ void st(float* p, f32x4 v) { *reinterpret_cast<f32x4*>(p) = v; }
+  static __device__ __forceinline__ float get(const f32x4& v, int j) { return v[j]; }
+  static __device__ __forceinline__ void set(f32x4& v, int j, float x) { v[j] = x; }
+};
+template <> struct Pack<bf16_t, 4> {
+  typedef f32x4 vec;
+  static __device__ __forceinline__ f32x4 ld(const bf16_t* p) {
+    const u16x4 r = *reinterpret_cast<const u16x4*>(p);
+    return f32x4{bf2f(r[0]), bf2f(r[1]), bf2f(r[2]), bf2f(r[3])};
+  }
+  static __device__ __forceinline__ void st(bf16_t* p, f32x4 v) {
+    *reinterpret_cast<u16x4*>(p) = u16x4{f2bf(v[0]), f2bf(v[1]), f2bf(v[2]), f2bf(v[3])};
+  }
+  static __device__ __forceinline__ float get(const f32x4& v, int j) { return v[j]; }
+  static __device__ __forceinline__ void set(f32x4& v, int j, float x) { v[j] = x; }
+};
+
 // Layer norm of the row staged in `u` (LDS, W floats, element i written by the thread that reads it).
-template <typename T>
+template <typename T, int V>
 __device__ __forceinline__ void layer_norm_row(const float* u, float part_sum, const float* __restrict__ w, float eps,
                                                T* __restrict__ out, int W, float* red) {
+  typedef Pack<float, V> PF;
   const float mean = block_sum(part_sum, red) / W;
   float sq = 0.f;
-  for (int i = threadIdx.x; i < W; i += NT) {
-    const float d = u[i] - mean;
-    sq += d * d;
+  for (int i = V * threadIdx.x; i < W; i += V * NT) {
+    const typename PF::vec x = PF::ld(u + i);
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      const float d = PF::get(x, j) - mean;
+      sq += d * d;
+    }
   }
   const float r = 1.0f / sqrtf(block_sum(sq, red) / W + eps);
-  for (int i = threadIdx.x; i < W; i += NT) out[i] = Elem<T>::st((u[i] - mean) * r * w[i]);
+  for (int i = V * threadIdx.x; i < W; i += V * NT) {
+    const typename PF::vec x = PF::ld(u + i), g = PF::ld(w + i);
+    typename PF::vec o;
+#pragma unroll
+    for (int j = 0; j < V; ++j) PF::set(o, j, (PF::get(x, j) - mean) * r * PF::get(g, j));
+    Pack<T, V>::st(out + i, o);
+  }
 }
 
 // X[t, s, :] = table[token] for every stream; h = layer_norm(sum_s r[s] X[s]).
@@ -77,12 +117,13 @@ __global__ __launch_bounds__(NT) void hyper_embed_norm_kernel(const int* __restr
     u[i] = acc;
     sum += acc;
   }
-  layer_norm_row<T>(u, sum, norm_w, eps, h + static_cast<size_t>(t) * W, W, red);
+  layer_norm_row<T, 1>(u, sum, norm_w, eps, h + static_cast<size_t>(t) * W, W, red);
 }
 
 // X'[t] = sum_s mix[s, t] X[s] + out_w[t] (y0 + y1) in place (mix null: X stays), then
-// h = layer_norm(sum_s read_w[s] X'[s]) (read_w null: no read).  SM >= S is the unrolled stream count.
-template <typename T, int SM>
+// h = layer_norm(sum_s read_w[s] X'[s]) (read_w null: no read).  SM >= S is the unrolled stream count,
+// V the columns per thread and access (4 when the width is a multiple of 4).
+template <typename T, int SM, int V>
 __global__ __launch_bounds__(NT) void hyper_update_norm_kernel(float* __restrict__ X, const T* __restrict__ y0,
                                                                const float* __restrict__ y1,
                                                                const float* __restrict__ mix,
@@ -90,9 +131,11 @@ __global__ __launch_bounds__(NT) void hyper_update_norm_kernel(float* __restrict
                                                                const float* __restrict__ read_w,
                                                                const float* __restrict__ norm_w, float eps,
                                                                T* __restrict__ h, int S, int W) {
-  extern __shared__ float u[];
+  extern __shared__ __attribute__((aligned(16))) float u[];
   __shared__ float red[NT / 64];
   __shared__ float cm[MAX_STREAMS * MAX_STREAMS], co[MAX_STREAMS], cr[MAX_STREAMS];
+  typedef Pack<float, V> PF;
+  typedef typename PF::vec vec;
   if (threadIdx.x < S * S) cm[threadIdx.x] = mix != nullptr ? mix[threadIdx.x] : 0.f;
   if (threadIdx.x < S) {
     co[threadIdx.x] = out_w != nullptr ? out_w[threadIdx.x] : 0.f;
@@ -102,30 +145,44 @@ __global__ __launch_bounds__(NT) void hyper_update_norm_kernel(float* __restrict
   const size_t t = blockIdx.x;
   float* x = X + t * S * W;
   float sum = 0.f;
-  for (int i = threadIdx.x; i < W; i += NT) {
-    float xs[SM], y = 0.f;
+  for (int i = V * threadIdx.x; i < W; i += V * NT) {
+    vec xs[SM], ya, yb, acc;
 #pragma unroll
-    for (int s = 0; s < SM; ++s) xs[s] = s < S ? x[static_cast<size_t>(s) * W + i] : 0.f;
-    if (y0 != nullptr) y += Elem<T>::ld(y0[t * W + i]);
-    if (y1 != nullptr) y += y1[t * W + i];
-    float acc = 0.f;
+    for (int s = 0; s < SM; ++s)
+      if (s < S) xs[s] = PF::ld(x + static_cast<size_t>(s) * W + i);
+    if (y0 != nullptr) ya = Pack<T, V>::ld(y0 + t * W + i);
+    if (y1 != nullptr) yb = PF::ld(y1 + t * W + i);
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      float y = 0.f;
+      if (y0 != nullptr) y += PF::get(ya, j);
+      if (y1 != nullptr) y += PF::get(yb, j);
+      PF::set(ya, j, y);
+      PF::set(acc, j, 0.f);
+    }
 #pragma unroll
     for (int d = 0; d < SM; ++d)
       if (d < S) {
-        float v = xs[d];
+        vec v = xs[d];
         if (mix != nullptr) {
-          v = co[d] * y;
 #pragma unroll
-          for (int s = 0; s < SM; ++s)
-            if (s < S) v += cm[s * S + d] * xs[s];
-          x[static_cast<size_t>(d) * W + i] = v;
+          for (int j = 0; j < V; ++j) {
+            float e = co[d] * PF::get(ya, j);
+#pragma unroll
+            for (int s = 0; s < SM; ++s)
+              if (s < S) e += cm[s * S + d] * PF::get(xs[s], j);
+            PF::set(v, j, e);
+          }
+          PF::st(x + static_cast<size_t>(d) * W + i, v);
         }
-        acc += cr[d] * v;
+#pragma unroll
+        for (int j = 0; j < V; ++j) PF::set(acc, j, PF::get(acc, j) + cr[d] * PF::get(v, j));
       }
-    u[i] = acc;
-    sum += acc;
+    PF::st(u + i, acc);
+#pragma unroll
+    for (int j = 0; j < V; ++j) sum += PF::get(acc, j);
   }
-  if (read_w != nullptr) layer_norm_row<T>(u, sum, norm_w, eps, h + t * W, W, red);
+  if (read_w != nullptr) layer_norm_row<T, V>(u, sum, norm_w, eps, h + t * W, W, red);
 }
 
 // One workgroup per token, a wave per q / k head: rotary on the first 2 half features (feature i
@@ -196,50 +253,58 @@ __global__ __launch_bounds__(NT) void rope_norm_kv_kernel(const T* __restrict__ 
   }
 }
 
-// q32 = q_scale * y[:, off_q + .], k32 = y[:, off_k + .] (fp32 copies of two column blocks of n features).
+// One workgroup per token: fp32 copies q32 = q_scale * y[off_q + .] and k32 = y[off_k + .] of two
+// column blocks of n features, and per head the log gates i = cap tanh((y_i + b_i) / cap) (into
+// `write`) and f = logsigmoid(cap tanh((y_f + b_f) / cap)) (into `decay`).
 template <typename T>
-__global__ __launch_bounds__(NT) void scaled_qk_kernel(const T* __restrict__ y, int64_t stride, int off_q, int off_k, int n,
-                                                       float q_scale, float* __restrict__ q32, float* __restrict__ k32,
-                                                       int64_t rows) {
-  const int64_t total = rows * n;
-  for (int64_t e = static_cast<int64_t>(blockIdx.x) * NT + threadIdx.x; e < total; e += static_cast<int64_t>(gridDim.x) * NT) {
-    const int64_t r = e / n;
-    const int c = static_cast<int>(e - r * n);
-    q32[e] = Elem<T>::ld(y[r * stride + off_q + c]) * q_scale;
-    k32[e] = Elem<T>::ld(y[r * stride + off_k + c]);
+__global__ __launch_bounds__(NT) void gate_rows_kernel(const T* __restrict__ y, int64_t stride, int off_q, int off_k, int off_i,
+                                                       int off_f, int n, float q_scale, const float* __restrict__ i_bias,
+                                                       const float* __restrict__ f_bias, float cap,
+                                                       float* __restrict__ q32, float* __restrict__ k32,
+                                                       float* __restrict__ decay, float* __restrict__ write, int H) {
+  const size_t t = blockIdx.x;
+  const T* row = y + t * stride;
+  for (int c = threadIdx.x; c < n; c += NT) {
+    q32[t * n + c] = Elem<T>::ld(row[off_q + c]) * q_scale;
+    k32[t * n + c] = Elem<T>::ld(row[off_k + c]);
+  }
+  const float inv = 1.0f / cap;
+  for (int h = threadIdx.x; h < H; h += NT) {
+    write[t * H + h] = cap * tanhf((Elem<T>::ld(row[off_i + h]) + i_bias[h]) * inv);
+    decay[t * H + h] = log_sigmoidf_(cap * tanhf((Elem<T>::ld(row[off_f + h]) + f_bias[h]) * inv));
   }
 }
 
-// One workgroup per segment, a thread per head.  The maximum is a chain of one add and one max
-// per token; the gates' tanh / logsigmoid before it and the three exponentials after it are
-// independent of the chain and are computed for CH tokens at a time around it.  The chain is the
-// same token by token whatever the segment's length, so a sequence's gates do not depend on how
-// it was cut.  m_state [n_rows, H] is read unless the segment starts at position 0.
-template <typename T, int CH>
-__global__ __launch_bounds__(NT) void gate_max_scan_kernel(const T* __restrict__ y, int64_t stride, int off_i, int off_f,
-                                                           const float* __restrict__ i_bias,
-                                                           const float* __restrict__ f_bias, float cap,
-                                                           const int* __restrict__ positions,
-                                                           const int* __restrict__ q_start,
-                                                           const int* __restrict__ state_rows,
-                                                           float* __restrict__ m_state, int n_rows,
-                                                           float* __restrict__ decay, float* __restrict__ write,
-                                                           float* __restrict__ floor_, int H) {
+// One workgroup per segment, a thread per head: the running maximum m_t = max(f_t + m_(t-1), i_t),
+// a chain of one add and one max per token over the log gates that `gate_rows_kernel` left in
+// `decay` (f) and `write` (i); they are replaced by the logarithms of what the recurrence needs,
+// f_t + m_(t-1) - m_t and i_t - m_t, and -m_t goes to `floor_`.  The next CH tokens' gates are
+// loaded while this chunk's chain runs.  The chain is the same token by token whatever the
+// segment's length, so a sequence's gates do not depend on how it was cut.  m_state [n_rows, H] is
+// read unless the segment starts at position 0.
+template <int CH>
+__global__ __launch_bounds__(NT) void gate_max_chain_kernel(const int* __restrict__ positions, const int* __restrict__ q_start,
+                                                            const int* __restrict__ state_rows, float* __restrict__ m_state,
+                                                            int n_rows, float* __restrict__ decay, float* __restrict__ write,
+                                                            float* __restrict__ floor_, int H) {
   const int b = blockIdx.x, h = threadIdx.x;
   const int t0 = q_start[b], t1 = q_start[b + 1];
   const int sr = state_rows[b];
   if (h >= H || t1 <= t0 || sr < 0 || sr >= n_rows) return;
   float m = positions[t0] != 0 ? m_state[static_cast<size_t>(sr) * H + h] : 0.f;
-  const float bi = i_bias[h], bf = f_bias[h], inv = 1.0f / cap;
-  for (int first = t0; first < t1; first += CH) {
-    float gi[CH], gf[CH], mm[CH + 1];
+  float gi[CH], gf[CH], ni[CH], nf[CH];
+  auto load = [&](int first, float (&a)[CH], float (&c)[CH]) {
 #pragma unroll
     for (int j = 0; j < CH; ++j) {
-      const int t = min(first + j, t1 - 1);
-      const T* row = y + static_cast<size_t>(t) * stride;
-      gi[j] = cap * tanhf((Elem<T>::ld(row[off_i + h]) + bi) * inv);
-      gf[j] = log_sigmoidf_(cap * tanhf((Elem<T>::ld(row[off_f + h]) + bf) * inv));
+      const size_t o = static_cast<size_t>(min(first + j, t1 - 1)) * H + h;
+      a[j] = write[o];
+      c[j] = decay[o];
     }
+  };
+  load(t0, gi, gf);
+  for (int first = t0; first < t1; first += CH) {
+    if (first + CH < t1) load(first + CH, ni, nf);
+    float mm[CH + 1];
     mm[0] = m;
 #pragma unroll
     for (int j = 0; j < CH; ++j) mm[j + 1] = fmaxf(gf[j] + mm[j], gi[j]);
@@ -248,14 +313,28 @@ __global__ __launch_bounds__(NT) void gate_max_scan_kernel(const T* __restrict__
       const int t = first + j;
       if (t < t1) {
         const size_t o = static_cast<size_t>(t) * H + h;
-        decay[o] = expf(gf[j] + mm[j] - mm[j + 1]);
-        write[o] = expf(gi[j] - mm[j + 1]);
-        floor_[o] = expf(-mm[j + 1]);
+        decay[o] = gf[j] + mm[j] - mm[j + 1];
+        write[o] = gi[j] - mm[j + 1];
+        floor_[o] = -mm[j + 1];
         m = mm[j + 1];
       }
     }
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+      gi[j] = ni[j];
+      gf[j] = nf[j];
+    }
   }
   m_state[static_cast<size_t>(sr) * H + h] = m;
+}
+
+// a, b, c <- exp(a), exp(b), exp(c) elementwise.
+__global__ __launch_bounds__(NT) void exp3_kernel(float* __restrict__ a, float* __restrict__ b, float* __restrict__ c, int64_t total) {
+  for (int64_t e = static_cast<int64_t>(blockIdx.x) * NT + threadIdx.x; e < total; e += static_cast<int64_t>(gridDim.x) * NT) {
+    a[e] = expf(a[e]);
+    b[e] = expf(b[e]);
+    c[e] = expf(c[e]);
+  }
 }
 
 // x <- cap tanh(x / cap) over fp32 logits.
@@ -271,10 +350,16 @@ template <typename T>
 int launch_update(float* X, const T* y0, const float* y1, const float* mix, const float* ow, const float* rw, const float* nw,
                   float eps, T* h, int T_, int S, int W, hipStream_t s) {
   const size_t lds = static_cast<size_t>(W) * sizeof(float);
-  if (S == 1) hyper_update_norm_kernel<T, 1><<<T_, NT, lds, s>>>(X, y0, y1, mix, ow, rw, nw, eps, h, S, W);
-  else if (S == 2) hyper_update_norm_kernel<T, 2><<<T_, NT, lds, s>>>(X, y0, y1, mix, ow, rw, nw, eps, h, S, W);
-  else if (S <= 4) hyper_update_norm_kernel<T, 4><<<T_, NT, lds, s>>>(X, y0, y1, mix, ow, rw, nw, eps, h, S, W);
-  else hyper_update_norm_kernel<T, 8><<<T_, NT, lds, s>>>(X, y0, y1, mix, ow, rw, nw, eps, h, S, W);
+#define BCG_UPDATE(SM_)                                                                                        \
+  do {                                                                                                         \
+    if (W % 4 == 0) hyper_update_norm_kernel<T, SM_, 4><<<T_, NT, lds, s>>>(X, y0, y1, mix, ow, rw, nw, eps, h, S, W); \
+    else hyper_update_norm_kernel<T, SM_, 1><<<T_, NT, lds, s>>>(X, y0, y1, mix, ow, rw, nw, eps, h, S, W);     \
+  } while (0)
+  if (S == 1) BCG_UPDATE(1);
+  else if (S == 2) BCG_UPDATE(2);
+  else if (S <= 4) BCG_UPDATE(4);
+  else BCG_UPDATE(8);
+#undef BCG_UPDATE
   return BCG_CHECK_LAUNCH();
 }
 
@@ -348,7 +433,8 @@ BCG_API int bcg_rope_norm_kv_write(const void* qkv, int64_t row_stride, const vo
                                   num_blocks, s);
 }
 
-// fp32 q (scaled) and k copies, then the gates and the running maximum of every (segment, head).
+// fp32 q (scaled) and k copies and the log gates per token, the running maximum of every (segment,
+// head), then the exponentials.
 BCG_API int bcg_exp_gate_prepare(const void* y, int64_t stride, int off_q, int off_k, int off_i, int off_f, const void* i_bias,
                                  const void* f_bias, float cap, float q_scale, const void* positions, const void* q_start,
                                  const void* state_rows, void* m_state, int n_rows, void* q32, void* k32, void* decay,
@@ -357,17 +443,16 @@ BCG_API int bcg_exp_gate_prepare(const void* y, int64_t stride, int off_q, int o
   if (H < 1 || H > NT || !(cap > 0.f)) return -2;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int n = H * dim;
-  const int64_t total = static_cast<int64_t>(T_) * n;
   const float *bi = static_cast<const float*>(i_bias), *bf = static_cast<const float*>(f_bias);
   const int *ps = static_cast<const int*>(positions), *qs = static_cast<const int*>(q_start), *sr = static_cast<const int*>(state_rows);
   float *q = static_cast<float*>(q32), *k = static_cast<float*>(k32), *m = static_cast<float*>(m_state),
         *dc = static_cast<float*>(decay), *wr = static_cast<float*>(write), *fl = static_cast<float*>(floor_);
-  BCG_BY_TYPE((scaled_qk_kernel<float><<<ew_grid(total), NT, 0, s>>>(static_cast<const float*>(y), stride, off_q, off_k, n, q_scale, q, k, T_)),
-              (scaled_qk_kernel<bf16_t><<<ew_grid(total), NT, 0, s>>>(static_cast<const bf16_t*>(y), stride, off_q, off_k, n, q_scale, q, k, T_)));
-  BCG_BY_TYPE((gate_max_scan_kernel<float, 16><<<B, NT, 0, s>>>(static_cast<const float*>(y), stride, off_i, off_f, bi, bf, cap, ps, qs, sr,
-                                                               m, n_rows, dc, wr, fl, H)),
-              (gate_max_scan_kernel<bf16_t, 16><<<B, NT, 0, s>>>(static_cast<const bf16_t*>(y), stride, off_i, off_f, bi, bf, cap, ps, qs,
-                                                                sr, m, n_rows, dc, wr, fl, H)));
+  BCG_BY_TYPE((gate_rows_kernel<float><<<T_, NT, 0, s>>>(static_cast<const float*>(y), stride, off_q, off_k, off_i, off_f, n, q_scale, bi, bf,
+                                                        cap, q, k, dc, wr, H)),
+              (gate_rows_kernel<bf16_t><<<T_, NT, 0, s>>>(static_cast<const bf16_t*>(y), stride, off_q, off_k, off_i, off_f, n, q_scale, bi,
+                                                         bf, cap, q, k, dc, wr, H)));
+  gate_max_chain_kernel<32><<<B, NT, 0, s>>>(ps, qs, sr, m, n_rows, dc, wr, fl, H);
+  exp3_kernel<<<ew_grid(static_cast<int64_t>(T_) * H), NT, 0, s>>>(dc, wr, fl, static_cast<int64_t>(T_) * H);
   return BCG_CHECK_LAUNCH();
 }
 
