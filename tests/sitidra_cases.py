@@ -67,6 +67,14 @@ CASES = {
 }
 
 
+# models of one kind of mixer: no K / V pages at all, no state tables at all
+ONE_KIND = {
+    "memories": config([layer("mlstm", mlstm(2, 16, 12)), layer("mlstm", mlstm(3, 8, 20, 3.0), 0)], width=40, streams=2),
+    "attention": config([layer("attention", attn(4, 4, 16, 16, 24, 8, v_mix=True), 0), layer("attention", attn(2, 1, 32, 8, 0, 32))],
+                        width=40, streams=2, softcap=0),
+}
+
+
 def checkpoint(cfg_dict, path, seed=0):
     """Write config.json + model.safetensors (bf16) under `path`; returns the tensors."""
     from safetensors.torch import save_file

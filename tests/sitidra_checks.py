@@ -299,8 +299,8 @@ def greedy_generation(env, cfg, sd, eng, tie=1e-3):
             seq.append(tok)
 
 
-def drawn_configuration(env, tmp_path, seed, pool_tokens=256):
-    cfg = C.random_config(seed)
+def drawn_configuration(env, tmp_path, seed, pool_tokens=256, cfg=None):
+    cfg = cfg or C.random_config(seed)
     path = str(tmp_path / "m")
     sd = O.to_f64(C.checkpoint(cfg, path, seed=seed))
     a, b = C.tokens(60, cfg["vocab"], seed), C.tokens(23, cfg["vocab"], seed + 100)

@@ -185,6 +185,11 @@ def test_drawn_configurations(tmp_path, seed):
     K.drawn_configuration(ENV, tmp_path, seed)
 
 
+@pytest.mark.parametrize("name", list(C.ONE_KIND))
+def test_models_of_one_kind_of_mixer(tmp_path, name):
+    K.drawn_configuration(ENV, tmp_path, 3, cfg=C.ONE_KIND[name])
+
+
 def test_text_entry_point_with_id_prompts(tmp_path):
     from byzantine_consensus_llm_agents_amd.engine import LLM, SamplingParams
     cfg = C.CASES["plain"]

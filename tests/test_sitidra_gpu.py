@@ -214,6 +214,12 @@ def test_drawn_configurations(tmp_path, seed, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", list(C.ONE_KIND))
+def test_models_of_one_kind_of_mixer(tmp_path, name, dtype):
+    K.drawn_configuration(K.Env("hip", "cuda", getattr(torch, dtype)), tmp_path, 3, cfg=C.ONE_KIND[name])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_long_context_chunks_across_decode_splits(tmp_path, dtype):
     """Chunks longer than a decode split and a context several chunks long: the decode kernel starts
     at the chunk's first split, the memories run hundreds of tokens."""
