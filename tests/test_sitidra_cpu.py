@@ -16,6 +16,7 @@ ENV = K.Env("torch", "cpu")
 @pytest.mark.parametrize("S", [1, 2, 3, 4, 7])
 def test_streams_read_write_and_layer_norm(S):
     K.check_streams(ENV, S)
+    K.check_streams(ENV, S, W=50)
 
 
 ATTENTION = {

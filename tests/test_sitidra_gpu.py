@@ -29,6 +29,8 @@ def env(request):
 def test_streams_read_write_and_layer_norm(env, S):
     K.check_streams(env, S)
     K.check_streams(env, S, W=1000)
+    K.check_streams(env, S, W=50)    # off the 4-column grid: one column per thread
+    K.check_streams(env, S, W=333)
 
 
 @pytest.mark.parametrize("name", list(ATTENTION))
@@ -108,7 +110,7 @@ def _tol(dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("S,W", [(4, 2048), (1, 96), (8, 1000), (2, 12288)])
+@pytest.mark.parametrize("S,W", [(4, 2048), (1, 96), (8, 1000), (2, 12288), (3, 1001), (4, 250)])
 def test_stream_kernels_at_model_widths(dtype, S, W):
     ops = K.Env("hip", "cuda").ops
     g = torch.Generator().manual_seed(S + W)
