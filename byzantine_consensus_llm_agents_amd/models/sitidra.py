@@ -230,7 +230,8 @@ class SitidraModel:
                     ups.append(pair(g, u) if pair else torch.cat([g, u]))
                 L["e_up"] = torch.stack(ups).contiguous()
                 L["e_down"] = torch.stack([get(p + f"mlp.e{e}.down") for e in range(f.experts)]).contiguous()
-                L["router"], L["correction"] = f32(p + "mlp.router"), f32(p + "mlp.correction")
+                L["router"] = f32(p + "mlp.router")
+                L["correction"] = f32(p + "mlp.correction") if p + "mlp.correction" in sd else None   # (none: the scores choose)
                 if f.shared_ff:
                     L["s_up"] = torch.cat([get(p + "mlp.shared.gate"), get(p + "mlp.shared.up")]).contiguous()
                     L["s_down"] = get(p + "mlp.shared.down")

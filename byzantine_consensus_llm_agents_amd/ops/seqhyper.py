@@ -12,7 +12,7 @@ import torch
 from .seqmix import _act, _check, _p, _req, _stream
 from .seqstate import _f32, _i32, _segments
 
-MAX_STREAMS = 8
+MAX_STREAMS = 16
 MAX_NORM_WIDTH = 12288
 
 
@@ -21,7 +21,7 @@ def seqhyper_ops(lib):
         _req(tokens.dtype == torch.int32 and tokens.is_contiguous() and tokens.dim() == 1, "tokens int32 [T]")
         _req(table.dim() == 2 and table.is_contiguous() and table.dtype == out_dtype, "table [V, W] in the activation dtype")
         T, W = tokens.numel(), table.shape[1]
-        _req(1 <= streams <= MAX_STREAMS and W <= MAX_NORM_WIDTH, "streams <= 8, width <= 12288")
+        _req(1 <= streams <= MAX_STREAMS and W <= MAX_NORM_WIDTH, "streams <= 16, width <= 12288")
         _f32(read_w, streams, "stream read weights")
         _f32(norm_w, W, "norm weight")
         X = torch.empty(T, streams, W, dtype=torch.float32, device=table.device)
@@ -33,7 +33,7 @@ def seqhyper_ops(lib):
     def hyper_update_norm(X, parts, mix, out_w, read_w, norm_w, eps, out_dtype):
         _req(X.dtype == torch.float32 and X.dim() == 3 and X.is_contiguous(), "streams fp32 [T, S, W]")
         T, S, W = X.shape
-        _req(1 <= S <= MAX_STREAMS and W <= MAX_NORM_WIDTH, "streams <= 8, width <= 12288")
+        _req(1 <= S <= MAX_STREAMS and W <= MAX_NORM_WIDTH, "streams <= 16, width <= 12288")
         typed = f32 = None
         for p in parts if mix is not None else ():
             _req(p.shape == (T, W) and p.is_contiguous(), "sublayer output [T, W] contiguous")

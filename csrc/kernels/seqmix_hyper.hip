@@ -21,7 +21,7 @@
 namespace {
 
 constexpr int NT = 256;
-constexpr int MAX_STREAMS = 8;
+constexpr int MAX_STREAMS = 16;
 
 __device__ __forceinline__ float block_sum(float v, float* red) {
   v = wave_sum(v);
@@ -358,7 +358,8 @@ int launch_update(float* X, const T* y0, const float* y1, const float* mix, cons
   if (S == 1) BCG_UPDATE(1);
   else if (S == 2) BCG_UPDATE(2);
   else if (S <= 4) BCG_UPDATE(4);
-  else BCG_UPDATE(8);
+  else if (S <= 8) BCG_UPDATE(8);
+  else BCG_UPDATE(16);
 #undef BCG_UPDATE
   return BCG_CHECK_LAUNCH();
 }

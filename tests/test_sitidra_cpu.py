@@ -13,7 +13,7 @@ ENV = K.Env("torch", "cpu")
 
 
 # ------------------------------------------------------------------ mechanisms
-@pytest.mark.parametrize("S", [1, 2, 3, 4, 7])
+@pytest.mark.parametrize("S", [1, 2, 3, 4, 7, 16])
 def test_streams_read_write_and_layer_norm(S):
     K.check_streams(ENV, S)
     K.check_streams(ENV, S, W=50)

@@ -25,7 +25,7 @@ def env(request):
 
 
 # ------------------------------------------------------------------ mechanisms
-@pytest.mark.parametrize("S", [1, 2, 3, 4, 7])
+@pytest.mark.parametrize("S", [1, 2, 3, 4, 7, 11, 16])
 def test_streams_read_write_and_layer_norm(env, S):
     K.check_streams(env, S)
     K.check_streams(env, S, W=1000)
