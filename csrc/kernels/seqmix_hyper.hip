@@ -275,66 +275,69 @@ __global__ __launch_bounds__(NT) void gate_rows_kernel(const T* __restrict__ y, 
   }
 }
 
-// One workgroup per segment, a thread per head: the running maximum m_t = max(f_t + m_(t-1), i_t),
-// a chain of one add and one max per token over the log gates that `gate_rows_kernel` left in
-// `decay` (f) and `write` (i); they are replaced by the logarithms of what the recurrence needs,
-// f_t + m_(t-1) - m_t and i_t - m_t, and -m_t goes to `floor_`.  The next CH tokens' gates are
-// loaded while this chunk's chain runs.  The chain is the same token by token whatever the
-// segment's length, so a sequence's gates do not depend on how it was cut.  m_state [n_rows, H] is
-// read unless the segment starts at position 0.
-template <int CH>
-__global__ __launch_bounds__(NT) void gate_max_chain_kernel(const int* __restrict__ positions, const int* __restrict__ q_start,
-                                                            const int* __restrict__ state_rows, float* __restrict__ m_state,
-                                                            int n_rows, float* __restrict__ decay, float* __restrict__ write,
-                                                            float* __restrict__ floor_, int H) {
-  const int b = blockIdx.x, h = threadIdx.x;
+constexpr int GATE_TILE = 4096;   // (token, head) pairs of a segment staged in LDS at a time
+
+// One workgroup per segment.  A tile of GATE_TILE / H tokens at a time: the workgroup stages the log
+// gates that `gate_rows_kernel` left in `write` (i) and `decay` (f) in LDS (coalesced loads); thread
+// h then walks the tile's tokens for head h, the running maximum m_t = max(f_t + m_(t-1), i_t) being
+// a chain of one add and one max per token, and leaves the logarithms f_t + m_(t-1) - m_t, i_t - m_t
+// and -m_t in LDS; every thread exponentiates them on the way out (decay, write scale, floor of the
+// denominator).  The chain is the same token by token
+// whatever the segment's length, so a sequence's gates do not depend on how it was cut.
+// m_state [n_rows, H] is read unless the segment starts at position 0.
+__global__ __launch_bounds__(NT) void gate_chain_kernel(const int* __restrict__ positions,
+                                                        const int* __restrict__ q_start, const int* __restrict__ state_rows,
+                                                        float* __restrict__ m_state, int n_rows, float* __restrict__ decay,
+                                                        float* __restrict__ write, float* __restrict__ floor_, int H) {
+  __shared__ float li[GATE_TILE], lf[GATE_TILE], lm[GATE_TILE];
+  const int b = blockIdx.x, tid = threadIdx.x;
   const int t0 = q_start[b], t1 = q_start[b + 1];
   const int sr = state_rows[b];
-  if (h >= H || t1 <= t0 || sr < 0 || sr >= n_rows) return;
-  float m = positions[t0] != 0 ? m_state[static_cast<size_t>(sr) * H + h] : 0.f;
-  float gi[CH], gf[CH], ni[CH], nf[CH];
-  auto load = [&](int first, float (&a)[CH], float (&c)[CH]) {
-#pragma unroll
-    for (int j = 0; j < CH; ++j) {
-      const size_t o = static_cast<size_t>(min(first + j, t1 - 1)) * H + h;
-      a[j] = write[o];
-      c[j] = decay[o];
+  if (t1 <= t0 || sr < 0 || sr >= n_rows) return;   // (the same for the whole workgroup)
+  const int tile = GATE_TILE / H;                  // tokens per tile
+  float m = 0.f;
+  if (tid < H && positions[t0] != 0) m = m_state[static_cast<size_t>(sr) * H + tid];
+  for (int first = t0; first < t1; first += tile) {
+    const int nt = min(tile, t1 - first), ne = nt * H;
+    const size_t base = static_cast<size_t>(first) * H;
+    for (int e = tid; e < ne; e += NT) {
+      li[e] = write[base + e];
+      lf[e] = decay[base + e];
     }
-  };
-  load(t0, gi, gf);
-  for (int first = t0; first < t1; first += CH) {
-    if (first + CH < t1) load(first + CH, ni, nf);
-    float mm[CH + 1];
-    mm[0] = m;
+    __syncthreads();
+    if (tid < H) {
+      constexpr int CH = 16;   // tokens read from LDS before their chain runs: the reads' latency is paid once per CH
+      for (int tt0 = 0; tt0 < nt; tt0 += CH) {
+        float gi[CH], gf[CH], mm[CH + 1];
 #pragma unroll
-    for (int j = 0; j < CH; ++j) mm[j + 1] = fmaxf(gf[j] + mm[j], gi[j]);
+        for (int j = 0; j < CH; ++j) {
+          const int e = min(tt0 + j, nt - 1) * H + tid;
+          gi[j] = li[e];
+          gf[j] = lf[e];
+        }
+        mm[0] = m;
 #pragma unroll
-    for (int j = 0; j < CH; ++j) {
-      const int t = first + j;
-      if (t < t1) {
-        const size_t o = static_cast<size_t>(t) * H + h;
-        decay[o] = gf[j] + mm[j] - mm[j + 1];
-        write[o] = gi[j] - mm[j + 1];
-        floor_[o] = -mm[j + 1];
-        m = mm[j + 1];
+        for (int j = 0; j < CH; ++j) mm[j + 1] = fmaxf(gf[j] + mm[j], gi[j]);
+#pragma unroll
+        for (int j = 0; j < CH; ++j)
+          if (tt0 + j < nt) {
+            const int e = (tt0 + j) * H + tid;
+            lf[e] = gf[j] + mm[j] - mm[j + 1];
+            li[e] = gi[j] - mm[j + 1];
+            lm[e] = -mm[j + 1];
+            m = mm[j + 1];
+          }
       }
     }
-#pragma unroll
-    for (int j = 0; j < CH; ++j) {
-      gi[j] = ni[j];
-      gf[j] = nf[j];
+    __syncthreads();
+    for (int e = tid; e < ne; e += NT) {
+      decay[base + e] = expf(lf[e]);
+      write[base + e] = expf(li[e]);
+      floor_[base + e] = expf(lm[e]);
     }
+    __syncthreads();
   }
-  m_state[static_cast<size_t>(sr) * H + h] = m;
-}
-
-// a, b, c <- exp(a), exp(b), exp(c) elementwise.
-__global__ __launch_bounds__(NT) void exp3_kernel(float* __restrict__ a, float* __restrict__ b, float* __restrict__ c, int64_t total) {
-  for (int64_t e = static_cast<int64_t>(blockIdx.x) * NT + threadIdx.x; e < total; e += static_cast<int64_t>(gridDim.x) * NT) {
-    a[e] = expf(a[e]);
-    b[e] = expf(b[e]);
-    c[e] = expf(c[e]);
-  }
+  if (tid < H) m_state[static_cast<size_t>(sr) * H + tid] = m;
 }
 
 // x <- cap tanh(x / cap) over fp32 logits.
@@ -434,8 +437,8 @@ BCG_API int bcg_rope_norm_kv_write(const void* qkv, int64_t row_stride, const vo
                                   num_blocks, s);
 }
 
-// fp32 q (scaled) and k copies and the log gates per token, the running maximum of every (segment,
-// head), then the exponentials.
+// fp32 q (scaled) and k copies and the log gates per token; then per segment the running maximum of
+// every head and the exponentials.
 BCG_API int bcg_exp_gate_prepare(const void* y, int64_t stride, int off_q, int off_k, int off_i, int off_f, const void* i_bias,
                                  const void* f_bias, float cap, float q_scale, const void* positions, const void* q_start,
                                  const void* state_rows, void* m_state, int n_rows, void* q32, void* k32, void* decay,
@@ -452,8 +455,7 @@ BCG_API int bcg_exp_gate_prepare(const void* y, int64_t stride, int off_q, int o
                                                         cap, q, k, dc, wr, H)),
               (gate_rows_kernel<bf16_t><<<T_, NT, 0, s>>>(static_cast<const bf16_t*>(y), stride, off_q, off_k, off_i, off_f, n, q_scale, bi,
                                                          bf, cap, q, k, dc, wr, H)));
-  gate_max_chain_kernel<32><<<B, NT, 0, s>>>(ps, qs, sr, m, n_rows, dc, wr, fl, H);
-  exp3_kernel<<<ew_grid(static_cast<int64_t>(T_) * H), NT, 0, s>>>(dc, wr, fl, static_cast<int64_t>(T_) * H);
+  gate_chain_kernel<<<B, NT, 0, s>>>(ps, qs, sr, m, n_rows, dc, wr, fl, H);
   return BCG_CHECK_LAUNCH();
 }
 
